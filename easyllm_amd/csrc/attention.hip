@@ -1,0 +1,587 @@
+// Causal, variable-length flash attention forward + backward for gfx950 (bf16 MFMA, fp32 softmax).
+//
+// Replaces the flash_attn_varlen_{qkv,kv}packed_func calls of the reference's FlashAttention
+// (llama/transformer.py:83-143): tokens are flattened to (b s); documents are the batch rows or the
+// cu_seqlens segments; attention is causal inside each document; softmax scale defaults to
+// 1/sqrt(d); query head i reads kv head i / (nq / nk) (MHA and GQA).
+//
+// Tensors are addressed as  token n -> (n / s_len) * batch_stride + (n % s_len) * seq_stride, heads
+// contiguous inside a token, so the [s, b, heads*d] activations of the layer are consumed and
+// produced in place (no [s,b]<->[b,s] copies, cf. transformer.py:478,491).
+//
+// All three kernels use the 32x32x16 bf16 MFMA with "transposed" score tiles so that the softmax
+// statistics of a query are per-lane scalars:
+//   forward       S^T = K Q^T (keys x queries), online softmax per lane, O^T += V^T P^T
+//   dK/dV kernel  S = Q K^T (queries x keys), dV^T += dO^T P, dK^T += Q^T dS   (block owns 128 keys)
+//   dQ kernel     S^T = K Q^T, dP^T = V dO^T, dQ^T += K^T dS^T                 (block owns 128 queries)
+// Operands whose reduction index is the strided one (V^T, K^T, Q^T, dO^T) are read from their
+// natural [row][d] LDS tiles with ds_read_b64_tr_b16; the accumulator registers of the score tile
+// are reused directly as the B operand of the second MFMA (the k index is permuted consistently).
+// LDS rows are padded to (d*2 + 48) bytes, which keeps both the 128-bit row reads and the transpose
+// reads free of bank conflicts.  K/V (or Q/dO) tiles are double buffered and filled through
+// registers one tile ahead.  dQ uses its own pass instead of atomics, so results are deterministic.
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
+
+struct AttnParams {
+    const bf16_t* q; const bf16_t* k; const bf16_t* v; const bf16_t* o; const bf16_t* dout;
+    bf16_t* out; bf16_t* dq; bf16_t* dk; bf16_t* dv;
+    float* lse; float* delta;
+    const int* cu;
+    int ndocs, s_len, T, nq, nk;
+    float scale;
+    int64_t q_ss, q_sb, k_ss, k_sb, v_ss, v_sb, o_ss, o_sb;          // forward tensors
+    int64_t do_ss, do_sb, dq_ss, dq_sb, dk_ss, dk_sb, dv_ss, dv_sb;  // backward tensors
+};
+
+__device__ __forceinline__ int64_t tok_off(int n, int s_len, int64_t ss, int64_t sb) {
+    const int b = n / s_len;
+    return (int64_t)b * sb + (int64_t)(n - b * s_len) * ss;
+}
+
+// block id -> (document, block inside the document); false if the id is beyond the last block
+__device__ __forceinline__ bool find_block(const int* __restrict__ cu, int ndocs, int s_len, int T, int bid, int blk_rows,
+                                           int& doc_start, int& doc_len, int& blk) {
+    for (int d = 0; d < ndocs; ++d) {
+        int a = cu ? cu[d] : d * s_len;
+        int e = cu ? cu[d + 1] : (d + 1) * s_len;
+        a = a < 0 ? 0 : a;
+        e = e > T ? T : e;
+        const int len = e - a;
+        if (len <= 0) continue;
+        const int nb = (len + blk_rows - 1) / blk_rows;
+        if (bid < nb) {
+            doc_start = a;
+            doc_len = len;
+            blk = bid;
+            return true;
+        }
+        bid -= nb;
+    }
+    return false;
+}
+
+template <int D>
+struct Tile {
+    static constexpr int LD = D + 24;             // padded row stride in elements
+    static constexpr int CH = D / 8;              // 128-bit chunks per row
+    static constexpr int ROWS = 64;
+    static constexpr int NCH = ROWS * CH / kThreads;  // chunks per thread
+    static constexpr int ELEMS = ROWS * LD;
+
+    // rows tok0 .. tok0+63 of head column hoff; rows at or beyond tok_end are zero
+    static __device__ __forceinline__ void load(const bf16_t* __restrict__ base, int64_t hoff, int tok0, int tok_end, int s_len,
+                                                int64_t ss, int64_t sb, int tid, bf16x8* r) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + kThreads * i;
+            const int row = c / CH, cc = c % CH;
+            const int n = tok0 + row;
+            bf16x8 z;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) z[j] = (bf16_t)0.0f;
+            r[i] = z;
+            if (n < tok_end) r[i] = *reinterpret_cast<const bf16x8*>(base + tok_off(n, s_len, ss, sb) + hoff + cc * 8);
+        }
+    }
+    static __device__ __forceinline__ void store(bf16_t* __restrict__ s, int tid, const bf16x8* r) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + kThreads * i;
+            *reinterpret_cast<bf16x8*>(s + (c / CH) * LD + (c % CH) * 8) = r[i];
+        }
+    }
+    // operand whose k index is d:   lane -> row (row0 + lane&31), d = kd*16 + 8*(lane>>5) ..+7
+    static __device__ __forceinline__ bf16x8 frag_kc(const bf16_t* __restrict__ s, int row0, int kd, int lane) {
+        return *reinterpret_cast<const bf16x8*>(s + (row0 + (lane & 31)) * LD + kd * 16 + (lane >> 5) * 8);
+    }
+    // operand whose k index is the tile row: lane -> d column (col0 + lane&31); k values are tile rows
+    // krow0 + 4g + {0..3} and krow0 + 8 + 4g + {0..3}, g = lane>>5 -- the order in which a 32x32
+    // accumulator block holds 16 consecutive rows, so accumulators convert straight to the B operand.
+    static __device__ __forceinline__ bf16x8 frag_tr(const bf16_t* __restrict__ s, int krow0, int col0, int lane) {
+        const int q = lane >> 4;
+        const bf16_t* p = s + (krow0 + 4 * (lane >> 5) + ((lane & 15) >> 2)) * LD + col0 + (q & 1) * 16 + ((lane & 3) << 2);
+        const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p));
+        const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p + 8 * LD));
+        bf16x8 v;
+        v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
+        v[4] = hi[0]; v[5] = hi[1]; v[6] = hi[2]; v[7] = hi[3];
+        return v;
+    }
+};
+
+// registers 8t .. 8t+7 of an accumulator block as a bf16 B operand
+__device__ __forceinline__ bf16x8 acc_to_b(const f32x16& a, int t) {
+    bf16x8 v;
+    if (t == 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (bf16_t)a[e];
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (bf16_t)a[8 + e];
+    }
+    return v;
+}
+
+// row of register r inside a 32-row accumulator block
+__device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+
+// one operand row per lane, straight from global memory, as D/16 B-operand fragments
+template <int D>
+__device__ __forceinline__ void load_row_frags(const bf16_t* __restrict__ rowp, int lane, bf16x8* f) {
+#pragma unroll
+    for (int kd = 0; kd < D / 16; ++kd) f[kd] = *reinterpret_cast<const bf16x8*>(rowp + kd * 16 + (lane >> 5) * 8);
+}
+
+// =================================================================================================
+// forward
+// =================================================================================================
+template <int D>
+__global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
+    using TL = Tile<D>;
+    __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS];  // K0 V0 K1 V1
+    int doc_start, doc_len, qb;
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, blockIdx.x, 128, doc_start, doc_len, qb)) return;
+    qb = (doc_len + 127) / 128 - 1 - qb;  // longest rows first
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hq = blockIdx.y, hk = hq / (p.nq / p.nk);
+    const int q0 = qb * 128, qw0 = q0 + wave * 32;
+    const int tok_end = doc_start + doc_len;
+    const int qi = qw0 + (lane & 31);                        // this lane's query (document relative)
+    const int qtok = doc_start + (qi < doc_len ? qi : doc_len - 1);
+    bf16x8 qf[D / 16];
+    load_row_frags<D>(p.q + tok_off(qtok, p.s_len, p.q_ss, p.q_sb) + (int64_t)hq * D, lane, qf);
+
+    const int kend = (q0 + 128 < doc_len ? q0 + 128 : doc_len);
+    const int ntiles = (kend + 63) / 64;
+    const int64_t kh = (int64_t)hk * D;
+    bf16x8 rk[TL::NCH], rv[TL::NCH];
+    TL::load(p.k, kh, doc_start, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
+    TL::load(p.v, kh, doc_start, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+    TL::store(smem, tid, rk);
+    TL::store(smem + TL::ELEMS, tid, rv);
+    if (ntiles > 1) {
+        TL::load(p.k, kh, doc_start + 64, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
+        TL::load(p.v, kh, doc_start + 64, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+    }
+    __syncthreads();
+
+    f32x16 oacc[D / 32];
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+    float m = -INFINITY, lsum = 0.f;
+    const float sl2 = p.scale * kLog2e;
+
+    for (int t = 0; t < ntiles; ++t) {
+        const int cur = t & 1;
+        const bf16_t* sK = smem + cur * 2 * TL::ELEMS;
+        const bf16_t* sV = sK + TL::ELEMS;
+        if (t + 1 < ntiles) {
+            TL::store(smem + (cur ^ 1) * 2 * TL::ELEMS, tid, rk);
+            TL::store(smem + (cur ^ 1) * 2 * TL::ELEMS + TL::ELEMS, tid, rv);
+        }
+        if (t + 2 < ntiles) {
+            TL::load(p.k, kh, doc_start + (t + 2) * 64, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
+            TL::load(p.v, kh, doc_start + (t + 2) * 64, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+        }
+        const int key0 = t * 64;
+        if (key0 <= qw0 + 31) {  // otherwise every key of the tile is after every query of this wave
+            f32x16 sacc[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+#pragma unroll
+                for (int kd = 0; kd < D / 16; ++kd)
+                    sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_kc(sK, kb * 32, kd, lane), qf[kd], sacc[kb], 0, 0, 0);
+            }
+            const bool need_mask = key0 + 63 > qw0;
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float s = sacc[kb][r] * sl2;
+                    if (need_mask && key0 + kb * 32 + acc_row(r, lane) > qi) s = -INFINITY;
+                    sacc[kb][r] = s;
+                    mloc = fmaxf(mloc, s);
+                }
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+            const float mnew = fmaxf(m, mloc);
+            const float msafe = mnew == -INFINITY ? 0.f : mnew;
+            const float alpha = __builtin_amdgcn_exp2f(m - msafe);
+            float psum = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float pe = __builtin_amdgcn_exp2f(sacc[kb][r] - msafe);
+                    sacc[kb][r] = pe;
+                    psum += pe;
+                }
+            lsum = lsum * alpha + psum;
+            m = mnew;
+#pragma unroll
+            for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    const bf16x8 pf = acc_to_b(sacc[kb], tt);
+#pragma unroll
+                    for (int db = 0; db < D / 32; ++db)
+                        oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_tr(sV, kb * 32 + 16 * tt, db * 32, lane), pf,
+                                                                           oacc[db], 0, 0, 0);
+                }
+        }
+        __syncthreads();
+    }
+    const float ltot = lsum + __shfl_xor(lsum, 32, 64);
+    if (qi < doc_len) {
+        const float inv = 1.0f / ltot;
+        bf16_t* orow = p.out + tok_off(doc_start + qi, p.s_len, p.o_ss, p.o_sb) + (int64_t)hq * D;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                bf16x4 w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = (bf16_t)(oacc[db][r4 * 4 + e] * inv);
+                *reinterpret_cast<bf16x4*>(orow + db * 32 + 8 * r4 + 4 * (lane >> 5)) = w;
+            }
+        if (lane < 32) p.lse[(int64_t)hq * p.T + doc_start + qi] = (m + __builtin_amdgcn_logf(ltot)) * kLn2;
+    }
+}
+
+// =================================================================================================
+// delta[h, n] = sum_d dO[n, h, d] * O[n, h, d]
+// =================================================================================================
+template <int D>
+__global__ __launch_bounds__(kThreads) void attn_delta_kernel(AttnParams p) {
+    constexpr int TPR = D / 8;  // threads per (token, head)
+    const int64_t items = (int64_t)p.T * p.nq;
+    const int sub = threadIdx.x % TPR;
+    // a (token, head) pair is owned by TPR consecutive lanes, which enter and leave the loop together
+    for (int64_t it = ((int64_t)blockIdx.x * kThreads + threadIdx.x) / TPR; it < items;
+         it += (int64_t)gridDim.x * (kThreads / TPR)) {
+        const int n = (int)(it / p.nq), h = (int)(it % p.nq);
+        float a[8], b[8], acc = 0.f;
+        unpack8(ld_bf16x8(p.o + tok_off(n, p.s_len, p.o_ss, p.o_sb) + (int64_t)h * D + sub * 8), a);
+        unpack8(ld_bf16x8(p.dout + tok_off(n, p.s_len, p.do_ss, p.do_sb) + (int64_t)h * D + sub * 8), b);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc += a[i] * b[i];
+#pragma unroll
+        for (int o = TPR / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+        if (sub == 0) p.delta[(int64_t)h * p.T + n] = acc;
+    }
+}
+
+// =================================================================================================
+// backward, dK and dV: a block owns 128 keys of one kv head and walks the queries at or after them
+// =================================================================================================
+template <int D>
+__global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
+    using TL = Tile<D>;
+    constexpr int STAGE = 2 * TL::ELEMS;                 // Q tile + dO tile
+    __shared__ __attribute__((aligned(16))) bf16_t smem[2 * STAGE];
+    __shared__ __attribute__((aligned(16))) float sstat[2][2][64];  // [stage][lse*log2e | delta][query]
+    int doc_start, doc_len, kbk;
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, blockIdx.x, 128, doc_start, doc_len, kbk)) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hk = blockIdx.y, group = p.nq / p.nk;
+    const int k0 = kbk * 128, kw0 = k0 + wave * 32;
+    const int tok_end = doc_start + doc_len;
+    const int kj = kw0 + (lane & 31);  // this lane's key (document relative)
+    const int ktok = doc_start + (kj < doc_len ? kj : doc_len - 1);
+    bf16x8 kf[D / 16], vf[D / 16];
+    load_row_frags<D>(p.k + tok_off(ktok, p.s_len, p.k_ss, p.k_sb) + (int64_t)hk * D, lane, kf);
+    load_row_frags<D>(p.v + tok_off(ktok, p.s_len, p.v_ss, p.v_sb) + (int64_t)hk * D, lane, vf);
+
+    f32x16 dkacc[D / 32], dvacc[D / 32];
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dkacc[i][r] = 0.f; dvacc[i][r] = 0.f; }
+
+    const int qt0 = k0 / 64;                      // first query tile that can see these keys
+    const int nqt = (doc_len + 63) / 64 - qt0;    // query tiles per head
+    const int total = nqt * group;                // flattened (head in group, query tile) iterations
+    const float sl2 = p.scale * kLog2e;
+
+    bf16x8 rq[TL::NCH], rdo[TL::NCH];
+    float rstat = 0.f;  // threads 0..63: lse*log2e of query tid; 64..127: delta of query tid-64
+    auto load_iter = [&](int it) {
+        const int hq = hk * group + it / nqt;
+        const int tok0 = doc_start + (qt0 + it % nqt) * 64;
+        TL::load(p.q, (int64_t)hq * D, tok0, tok_end, p.s_len, p.q_ss, p.q_sb, tid, rq);
+        TL::load(p.dout, (int64_t)hq * D, tok0, tok_end, p.s_len, p.do_ss, p.do_sb, tid, rdo);
+        if (tid < 128) {
+            const int n = tok0 + (tid & 63);
+            rstat = 0.f;
+            if (n < tok_end) rstat = tid < 64 ? p.lse[(int64_t)hq * p.T + n] * kLog2e : p.delta[(int64_t)hq * p.T + n];
+        }
+    };
+    auto store_iter = [&](int stage) {
+        TL::store(smem + stage * STAGE, tid, rq);
+        TL::store(smem + stage * STAGE + TL::ELEMS, tid, rdo);
+        if (tid < 128) sstat[stage][tid >> 6][tid & 63] = rstat;
+    };
+    load_iter(0);
+    store_iter(0);
+    if (total > 1) load_iter(1);
+    __syncthreads();
+
+    for (int it = 0; it < total; ++it) {
+        const int cur = it & 1;
+        const bf16_t* sQ = smem + cur * STAGE;
+        const bf16_t* sdO = sQ + TL::ELEMS;
+        if (it + 1 < total) store_iter(cur ^ 1);
+        if (it + 2 < total) load_iter(it + 2);
+        const int qbase = (qt0 + it % nqt) * 64;
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            const int qs0 = qbase + sub * 32;
+            if (qs0 + 31 < kw0 || qs0 >= doc_len) continue;  // all queries before this wave's keys / past the end
+            f32x16 sacc, dpacc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
+#pragma unroll
+            for (int kd = 0; kd < D / 16; ++kd) {
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_kc(sQ, sub * 32, kd, lane), kf[kd], sacc, 0, 0, 0);
+                dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_kc(sdO, sub * 32, kd, lane), vf[kd], dpacc, 0, 0, 0);
+            }
+            // accumulator register r <-> query qs0 + acc_row(r); lane <-> key kj
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int ql = sub * 32 + 8 * r4 + 4 * (lane >> 5);
+                const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sstat[cur][0][ql]);
+                const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sstat[cur][1][ql]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int r = r4 * 4 + e;
+                    const int qidx = qbase + ql + e;
+                    float pe = __builtin_amdgcn_exp2f(sacc[r] * sl2 - l4[e]);
+                    if (kj > qidx || qidx >= doc_len) pe = 0.f;
+                    sacc[r] = pe;
+                    dpacc[r] = pe * (dpacc[r] - d4[e]);
+                }
+            }
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                const bf16x8 pf = acc_to_b(sacc, tt);
+                const bf16x8 dsf = acc_to_b(dpacc, tt);
+#pragma unroll
+                for (int db = 0; db < D / 32; ++db) {
+                    dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_tr(sdO, sub * 32 + 16 * tt, db * 32, lane), pf,
+                                                                        dvacc[db], 0, 0, 0);
+                    dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_tr(sQ, sub * 32 + 16 * tt, db * 32, lane), dsf,
+                                                                        dkacc[db], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (kj < doc_len) {
+        bf16_t* dkrow = p.dk + tok_off(doc_start + kj, p.s_len, p.dk_ss, p.dk_sb) + (int64_t)hk * D;
+        bf16_t* dvrow = p.dv + tok_off(doc_start + kj, p.s_len, p.dv_ss, p.dv_sb) + (int64_t)hk * D;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                bf16x4 a, b;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    a[e] = (bf16_t)(dkacc[db][r4 * 4 + e] * p.scale);
+                    b[e] = (bf16_t)dvacc[db][r4 * 4 + e];
+                }
+                const int dcol = db * 32 + 8 * r4 + 4 * (lane >> 5);
+                *reinterpret_cast<bf16x4*>(dkrow + dcol) = a;
+                *reinterpret_cast<bf16x4*>(dvrow + dcol) = b;
+            }
+    }
+}
+
+// =================================================================================================
+// backward, dQ: a block owns 128 queries of one head and walks the keys at or before them
+// =================================================================================================
+template <int D>
+__global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(AttnParams p) {
+    using TL = Tile<D>;
+    __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS];  // K0 V0 K1 V1
+    int doc_start, doc_len, qb;
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, blockIdx.x, 128, doc_start, doc_len, qb)) return;
+    qb = (doc_len + 127) / 128 - 1 - qb;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hq = blockIdx.y, hk = hq / (p.nq / p.nk);
+    const int q0 = qb * 128, qw0 = q0 + wave * 32;
+    const int tok_end = doc_start + doc_len;
+    const int qi = qw0 + (lane & 31);
+    const int qtok = doc_start + (qi < doc_len ? qi : doc_len - 1);
+    bf16x8 qf[D / 16], dof[D / 16];
+    load_row_frags<D>(p.q + tok_off(qtok, p.s_len, p.q_ss, p.q_sb) + (int64_t)hq * D, lane, qf);
+    load_row_frags<D>(p.dout + tok_off(qtok, p.s_len, p.do_ss, p.do_sb) + (int64_t)hq * D, lane, dof);
+    const float lse2 = p.lse[(int64_t)hq * p.T + qtok] * kLog2e;
+    const float dlt = p.delta[(int64_t)hq * p.T + qtok];
+
+    const int kend = (q0 + 128 < doc_len ? q0 + 128 : doc_len);
+    const int ntiles = (kend + 63) / 64;
+    const int64_t kh = (int64_t)hk * D;
+    bf16x8 rk[TL::NCH], rv[TL::NCH];
+    TL::load(p.k, kh, doc_start, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
+    TL::load(p.v, kh, doc_start, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+    TL::store(smem, tid, rk);
+    TL::store(smem + TL::ELEMS, tid, rv);
+    if (ntiles > 1) {
+        TL::load(p.k, kh, doc_start + 64, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
+        TL::load(p.v, kh, doc_start + 64, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+    }
+    __syncthreads();
+
+    f32x16 dqacc[D / 32];
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dqacc[i][r] = 0.f;
+    const float sl2 = p.scale * kLog2e;
+
+    for (int t = 0; t < ntiles; ++t) {
+        const int cur = t & 1;
+        const bf16_t* sK = smem + cur * 2 * TL::ELEMS;
+        const bf16_t* sV = sK + TL::ELEMS;
+        if (t + 1 < ntiles) {
+            TL::store(smem + (cur ^ 1) * 2 * TL::ELEMS, tid, rk);
+            TL::store(smem + (cur ^ 1) * 2 * TL::ELEMS + TL::ELEMS, tid, rv);
+        }
+        if (t + 2 < ntiles) {
+            TL::load(p.k, kh, doc_start + (t + 2) * 64, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
+            TL::load(p.v, kh, doc_start + (t + 2) * 64, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+        }
+        const int key0 = t * 64;
+        if (key0 <= qw0 + 31) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                f32x16 sacc, dpacc;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
+#pragma unroll
+                for (int kd = 0; kd < D / 16; ++kd) {
+                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_kc(sK, kb * 32, kd, lane), qf[kd], sacc, 0, 0, 0);
+                    dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_kc(sV, kb * 32, kd, lane), dof[kd], dpacc, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float pe = __builtin_amdgcn_exp2f(sacc[r] * sl2 - lse2);
+                    if (key0 + kb * 32 + acc_row(r, lane) > qi) pe = 0.f;
+                    dpacc[r] = pe * (dpacc[r] - dlt);
+                }
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    const bf16x8 dsf = acc_to_b(dpacc, tt);
+#pragma unroll
+                    for (int db = 0; db < D / 32; ++db)
+                        dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_tr(sK, kb * 32 + 16 * tt, db * 32, lane), dsf,
+                                                                            dqacc[db], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (qi < doc_len) {
+        bf16_t* dqrow = p.dq + tok_off(doc_start + qi, p.s_len, p.dq_ss, p.dq_sb) + (int64_t)hq * D;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                bf16x4 w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = (bf16_t)(dqacc[db][r4 * 4 + e] * p.scale);
+                *reinterpret_cast<bf16x4*>(dqrow + db * 32 + 8 * r4 + 4 * (lane >> 5)) = w;
+            }
+    }
+}
+
+int check_common(const char* name, int64_t T, int64_t s_len, int64_t nq, int64_t nk, int64_t d, int64_t ndocs, const int64_t* strides,
+                 int nstrides) {
+    EZL_REQUIRE(d == 64 || d == 128, EZL_EUNSUPPORTED, "%s: head dim must be 64 or 128 (got %lld)", name, (long long)d);
+    EZL_REQUIRE(nq > 0 && nk > 0 && nq % nk == 0, EZL_EINVAL, "%s: nq must be a positive multiple of nk", name);
+    EZL_REQUIRE(T >= 0 && T < (1LL << 30) && s_len > 0 && T % s_len == 0 && ndocs > 0 && ndocs < (1LL << 24), EZL_EINVAL,
+                "%s: bad token / document counts", name);
+    EZL_REQUIRE(nq < 65536, EZL_EUNSUPPORTED, "%s: too many heads", name);
+    for (int i = 0; i < nstrides; ++i) EZL_REQUIRE(strides[i] % 8 == 0, EZL_EINVAL, "%s: strides must be multiples of 8 elements", name);
+    return EZL_OK;
+}
+
+}  // namespace
+
+// strides[8]: q_seq, q_batch, k_seq, k_batch, v_seq, v_batch, out_seq, out_batch (elements)
+extern "C" int ezl_attn_fwd(const void* q, const void* k, const void* v, void* out, void* lse, const void* cu_seqlens, int64_t ndocs,
+                            int64_t total_tokens, int64_t s_len, int64_t nq, int64_t nk, int64_t d, float scale,
+                            const int64_t* strides, void* stream) {
+    int rc = check_common("ezl_attn_fwd", total_tokens, s_len, nq, nk, d, ndocs, strides, 8);
+    if (rc) return rc;
+    if (total_tokens == 0) return EZL_OK;
+    EZL_REQUIRE(q && k && v && out && lse && ezl_aligned16(q) && ezl_aligned16(k) && ezl_aligned16(v) && ezl_aligned16(out), EZL_EINVAL,
+                "ezl_attn_fwd: null or misaligned pointer");
+    AttnParams p = {};
+    p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.v = (const bf16_t*)v; p.out = (bf16_t*)out; p.lse = (float*)lse;
+    p.cu = (const int*)cu_seqlens; p.ndocs = (int)ndocs; p.s_len = (int)s_len; p.T = (int)total_tokens; p.nq = (int)nq; p.nk = (int)nk;
+    p.scale = scale;
+    p.q_ss = strides[0]; p.q_sb = strides[1]; p.k_ss = strides[2]; p.k_sb = strides[3];
+    p.v_ss = strides[4]; p.v_sb = strides[5]; p.o_ss = strides[6]; p.o_sb = strides[7];
+    const dim3 grid((unsigned)((total_tokens + 127) / 128 + ndocs), (unsigned)nq);
+    if (d == 128) hipLaunchKernelGGL(attn_fwd_kernel<128>, grid, dim3(kThreads), 0, (hipStream_t)stream, p);
+    else hipLaunchKernelGGL(attn_fwd_kernel<64>, grid, dim3(kThreads), 0, (hipStream_t)stream, p);
+    EZL_LAUNCH_CHECK("ezl_attn_fwd");
+    return EZL_OK;
+}
+
+// strides[16]: q, k, v, out (as above), then dout, dq, dk, dv (seq, batch each)
+extern "C" int ezl_attn_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout, const void* lse,
+                            void* delta, void* dq, void* dk, void* dv, const void* cu_seqlens, int64_t ndocs, int64_t total_tokens,
+                            int64_t s_len, int64_t nq, int64_t nk, int64_t d, float scale, const int64_t* strides, void* stream) {
+    int rc = check_common("ezl_attn_bwd", total_tokens, s_len, nq, nk, d, ndocs, strides, 16);
+    if (rc) return rc;
+    if (total_tokens == 0) return EZL_OK;
+    EZL_REQUIRE(q && k && v && out && dout && lse && delta && dq && dk && dv, EZL_EINVAL, "ezl_attn_bwd: null pointer");
+    EZL_REQUIRE(ezl_aligned16(q) && ezl_aligned16(k) && ezl_aligned16(v) && ezl_aligned16(out) && ezl_aligned16(dout) &&
+                    ezl_aligned16(dq) && ezl_aligned16(dk) && ezl_aligned16(dv),
+                EZL_EINVAL, "ezl_attn_bwd: misaligned pointer");
+    AttnParams p = {};
+    p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.v = (const bf16_t*)v; p.o = (const bf16_t*)out; p.dout = (const bf16_t*)dout;
+    p.lse = (float*)const_cast<void*>(lse); p.delta = (float*)delta; p.dq = (bf16_t*)dq; p.dk = (bf16_t*)dk; p.dv = (bf16_t*)dv;
+    p.cu = (const int*)cu_seqlens; p.ndocs = (int)ndocs; p.s_len = (int)s_len; p.T = (int)total_tokens; p.nq = (int)nq; p.nk = (int)nk;
+    p.scale = scale;
+    p.q_ss = strides[0]; p.q_sb = strides[1]; p.k_ss = strides[2]; p.k_sb = strides[3];
+    p.v_ss = strides[4]; p.v_sb = strides[5]; p.o_ss = strides[6]; p.o_sb = strides[7];
+    p.do_ss = strides[8]; p.do_sb = strides[9]; p.dq_ss = strides[10]; p.dq_sb = strides[11];
+    p.dk_ss = strides[12]; p.dk_sb = strides[13]; p.dv_ss = strides[14]; p.dv_sb = strides[15];
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t items = total_tokens * nq;
+    const int per_block = kThreads / (int)(d / 8);
+    int64_t g = (items + per_block - 1) / per_block;
+    if (g > 256 * 32) g = 256 * 32;
+    const dim3 gridq((unsigned)((total_tokens + 127) / 128 + ndocs), (unsigned)nq);
+    const dim3 gridk((unsigned)((total_tokens + 127) / 128 + ndocs), (unsigned)nk);
+    if (d == 128) {
+        hipLaunchKernelGGL(attn_delta_kernel<128>, dim3((unsigned)g), dim3(kThreads), 0, st, p);
+        hipLaunchKernelGGL(attn_bwd_dkdv_kernel<128>, gridk, dim3(kThreads), 0, st, p);
+        hipLaunchKernelGGL(attn_bwd_dq_kernel<128>, gridq, dim3(kThreads), 0, st, p);
+    } else {
+        hipLaunchKernelGGL(attn_delta_kernel<64>, dim3((unsigned)g), dim3(kThreads), 0, st, p);
+        hipLaunchKernelGGL(attn_bwd_dkdv_kernel<64>, gridk, dim3(kThreads), 0, st, p);
+        hipLaunchKernelGGL(attn_bwd_dq_kernel<64>, gridq, dim3(kThreads), 0, st, p);
+    }
+    EZL_LAUNCH_CHECK("ezl_attn_bwd");
+    return EZL_OK;
+}

@@ -1,0 +1,76 @@
+// Shared device/host helpers for the gfx950 kernels of the llama decoder-layer step.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+typedef __bf16 bf16_t;
+typedef bf16_t bf16x2 __attribute__((ext_vector_type(2)));
+typedef bf16_t bf16x4 __attribute__((ext_vector_type(4)));
+typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define EZL_OK 0
+#define EZL_EINVAL (-1)
+#define EZL_EUNSUPPORTED (-2)
+#define EZL_EHIP (-3)
+
+#define EZL_WAVE 64
+
+// thread-local last-error text, read back through ezl_last_error()
+void ezl_set_error(const char* fmt, ...);
+
+#define EZL_REQUIRE(cond, code, ...)      \
+    do {                                  \
+        if (!(cond)) {                    \
+            ezl_set_error(__VA_ARGS__);   \
+            return (code);                \
+        }                                 \
+    } while (0)
+
+// surfaces launch-configuration errors without synchronising the device
+#define EZL_LAUNCH_CHECK(name)                                                     \
+    do {                                                                           \
+        hipError_t e__ = hipGetLastError();                                        \
+        if (e__ != hipSuccess) {                                                   \
+            ezl_set_error("%s: launch failed: %s", (name), hipGetErrorString(e__)); \
+            return EZL_EHIP;                                                       \
+        }                                                                          \
+    } while (0)
+
+static inline bool ezl_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+#ifdef __HIPCC__
+// 8 bf16 <-> 8 fp32 (one 128-bit HBM transaction per lane)
+struct alignas(16) bf16x8_raw {
+    bf16x8 v;
+};
+
+__device__ __forceinline__ bf16x8 ld_bf16x8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ void st_bf16x8(bf16_t* p, bf16x8 v) { *reinterpret_cast<bf16x8*>(p) = v; }
+
+__device__ __forceinline__ void unpack8(bf16x8 v, float* f) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
+}
+__device__ __forceinline__ bf16x8 pack8(const float* f) {
+    bf16x8 v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (bf16_t)f[i];
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+#endif

@@ -1,0 +1,342 @@
+// Vocab-parallel cross entropy at TP=1 for gfx950 (HBM-bound).
+//
+// Restates base_modules/functions/cross_entropy.py:24-112 and llama/losses.py:20-56 of the
+// reference without its fp32 [T, V] copy and ~10 passes:
+//   * ezl_ce_prepare      weights w = loss_mask * (label != -100) and N = sum(w)      (losses.py:21-23,45)
+//   * ezl_ce_fwd          per-token loss + logsumexp                                  (cross_entropy.py:24-89)
+//   * ezl_ce_bwd          (softmax - onehot[valid]) * grad_out                        (cross_entropy.py:91-112)
+//   * ezl_ce_fused        loss rows AND d loss / d logits in one visit of the logits, for the
+//                         mean-reduced loss: grad = (softmax - onehot) * w / N
+//   * ezl_ce_reduce       loss = sum(loss_row * w) / N                                (losses.py:55)
+// A row of logits (bf16 or fp32) is owned by one 512-thread block.  When the row fits 64 KiB of
+// LDS it is staged there during the max pass, so HBM sees one read and (for bwd/fused) one write.
+// Integer semantics are exact: a label outside [0, V - cut) is "masked": pred = 0, no one-hot.
+#include "common.h"
+
+namespace {
+
+constexpr int kCeBlock = 512;
+constexpr int kCeWaves = kCeBlock / 64;
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <typename T> struct Vec8;
+template <> struct Vec8<bf16_t> {
+    static __device__ __forceinline__ void load(const bf16_t* p, float* f) { unpack8(ld_bf16x8(p), f); }
+    static __device__ __forceinline__ void store(bf16_t* p, const float* f) { st_bf16x8(p, pack8(f)); }
+};
+template <> struct Vec8<float> {
+    static __device__ __forceinline__ void load(const float* p, float* f) {
+        const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+        f[0] = a[0]; f[1] = a[1]; f[2] = a[2]; f[3] = a[3]; f[4] = b[0]; f[5] = b[1]; f[6] = b[2]; f[7] = b[3];
+    }
+    static __device__ __forceinline__ void store(float* p, const float* f) {
+        f32x4 a = {f[0], f[1], f[2], f[3]}, b = {f[4], f[5], f[6], f[7]};
+        *reinterpret_cast<f32x4*>(p) = a;
+        *reinterpret_cast<f32x4*>(p + 4) = b;
+    }
+};
+
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    __syncthreads();  // red may still be read from the previous reduction
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int i = 1; i < kCeWaves; ++i) r = fmaxf(r, red[i]);
+    return r;
+}
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = 0.f;
+#pragma unroll
+    for (int i = 0; i < kCeWaves; ++i) r += red[i];
+    return r;
+}
+
+// Max and sum(exp(x - max)) over columns [0, vend) of one row; optionally stages the row in LDS.
+template <typename T, bool IN_LDS>
+__device__ __forceinline__ void row_max_sumexp(const T* __restrict__ xrow, T* __restrict__ srow, int V, int vend, float* red,
+                                               float& m_out, float& s_out) {
+    const int v8 = V >> 3;
+    float m = -INFINITY;
+    for (int i = threadIdx.x; i < v8; i += kCeBlock) {
+        float f[8];
+        Vec8<T>::load(xrow + i * 8, f);
+        if (IN_LDS) Vec8<T>::store(srow + i * 8, f);
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (i * 8 + k < vend) m = fmaxf(m, f[k]);
+    }
+    m = block_max(m, red);  // barriers inside also publish the staged row
+    float s = 0.f;
+    const float mb = m * kLog2e;
+    for (int i = threadIdx.x; i < v8; i += kCeBlock) {
+        float f[8];
+        Vec8<T>::load((IN_LDS ? (const T*)srow : xrow) + i * 8, f);
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (i * 8 + k < vend) s += exp2f(f[k] * kLog2e - mb);
+    }
+    s = block_sum(s, red);
+    m_out = m;
+    s_out = s;
+}
+
+// grad[c] = (exp(x[c] - lse) - [c == target]) * scale   for every column (cut columns included)
+template <typename T, bool IN_LDS>
+__device__ __forceinline__ void row_write_grad(const T* __restrict__ xrow, const T* __restrict__ srow, T* __restrict__ grow,
+                                               int V, float lse, int target, float scale) {
+    const int v8 = V >> 3;
+    const float lb = lse * kLog2e;
+    for (int i = threadIdx.x; i < v8; i += kCeBlock) {
+        float f[8];
+        Vec8<T>::load((IN_LDS ? srow : xrow) + i * 8, f);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            float p = exp2f(f[k] * kLog2e - lb);
+            if (i * 8 + k == target) p -= 1.0f;
+            f[k] = p * scale;
+        }
+        Vec8<T>::store(grow + i * 8, f);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void row_write_zero(T* __restrict__ grow, int V) {
+    float z[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int i = threadIdx.x; i < (V >> 3); i += kCeBlock) Vec8<T>::store(grow + i * 8, z);
+}
+
+template <typename T, bool IN_LDS>
+__global__ __launch_bounds__(kCeBlock) void ce_fwd_kernel(const T* __restrict__ logits, const int64_t* __restrict__ labels,
+                                                          float* __restrict__ loss, float* __restrict__ lse_out, int64_t rows,
+                                                          int V, int vend) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    __shared__ float red[kCeWaves];
+    T* srow = reinterpret_cast<T*>(smem_raw);
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+        const T* xrow = logits + r * V;
+        float m, s;
+        row_max_sumexp<T, IN_LDS>(xrow, srow, V, vend, red, m, s);
+        if (threadIdx.x == 0) {
+            const int64_t t = labels[r];
+            const bool masked = t < 0 || t >= vend;
+            const float pred = masked ? 0.f : ((float)xrow[t] - m);  // cross_entropy.py:58-65 (shifted logit)
+            loss[r] = logf(s) - pred;                                // :83
+            lse_out[r] = m + logf(s);
+        }
+        __syncthreads();  // the staged row is overwritten by the next iteration
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kCeBlock) void ce_bwd_kernel(const T* __restrict__ logits, const int64_t* __restrict__ labels,
+                                                          const float* __restrict__ lse, const float* __restrict__ grad_out,
+                                                          T* __restrict__ grad, int64_t rows, int V, int vend) {
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+        const int64_t t = labels[r];
+        const int target = (t < 0 || t >= vend) ? -1 : (int)t;
+        row_write_grad<T, false>(logits + r * V, nullptr, grad + r * V, V, lse[r], target, grad_out[r]);
+    }
+}
+
+template <typename T, bool IN_LDS>
+__global__ __launch_bounds__(kCeBlock) void ce_fused_kernel(const T* __restrict__ logits, const int64_t* __restrict__ labels,
+                                                            const float* __restrict__ weights, const float* __restrict__ count,
+                                                            float* __restrict__ loss, T* __restrict__ grad, int64_t rows, int V,
+                                                            int vend) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    __shared__ float red[kCeWaves];
+    T* srow = reinterpret_cast<T*>(smem_raw);
+    const float inv_n = 1.0f / count[0];
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+        const float w = weights[r];
+        T* grow = grad + r * V;
+        if (w == 0.f) {  // ignored position: exact zero gradient, contributes nothing to the loss
+            row_write_zero<T>(grow, V);
+            if (threadIdx.x == 0) loss[r] = 0.f;
+            continue;
+        }
+        const T* xrow = logits + r * V;
+        const int64_t t = labels[r];
+        const bool masked = t < 0 || t >= vend;
+        // read the target logit before the row is overwritten in place
+        const float xt = masked ? 0.f : (float)xrow[t];
+        float m, s;
+        row_max_sumexp<T, IN_LDS>(xrow, srow, V, vend, red, m, s);
+        const float lse = m + logf(s);
+        if (threadIdx.x == 0) loss[r] = masked ? logf(s) : (lse - xt);
+        row_write_grad<T, IN_LDS>(xrow, srow, grow, V, lse, masked ? -1 : (int)t, w * inv_n);
+        __syncthreads();
+    }
+}
+
+// weights[i] = mask[i] * (labels[i] != ignore_index); count[0] = sum(weights) -- one block, fixed order
+__global__ __launch_bounds__(1024) void ce_prepare_kernel(const int64_t* __restrict__ labels, const void* __restrict__ mask,
+                                                          int mask_dtype, int64_t ignore_index, float* __restrict__ weights,
+                                                          float* __restrict__ count, int64_t n) {
+    __shared__ float red[16];
+    float acc = 0.f;
+    for (int64_t i = threadIdx.x; i < n; i += 1024) {
+        float mv = 1.0f;
+        if (mask_dtype == 1) mv = reinterpret_cast<const float*>(mask)[i];
+        else if (mask_dtype == 2) mv = reinterpret_cast<const unsigned char*>(mask)[i] ? 1.0f : 0.0f;
+        else if (mask_dtype == 3) mv = (float)reinterpret_cast<const int64_t*>(mask)[i];
+        else if (mask_dtype == 4) mv = (float)reinterpret_cast<const bf16_t*>(mask)[i];
+        const float w = labels[i] != ignore_index ? mv : 0.0f;
+        weights[i] = w;
+        acc += w;
+    }
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.f;
+        for (int i = 0; i < 16; ++i) t += red[i];
+        count[0] = t;
+    }
+}
+
+// out[0] = sum(loss[i] * weights[i]) / count[0]
+__global__ __launch_bounds__(1024) void ce_reduce_kernel(const float* __restrict__ loss, const float* __restrict__ weights,
+                                                         const float* __restrict__ count, float* __restrict__ out, int64_t n) {
+    __shared__ float red[16];
+    float acc = 0.f;
+    for (int64_t i = threadIdx.x; i < n; i += 1024) acc += loss[i] * weights[i];
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = 0.f;
+        for (int i = 0; i < 16; ++i) t += red[i];
+        out[0] = t / count[0];
+    }
+}
+
+// x[i] *= s[0] unless s[0] == 1 (the usual case for loss.backward(): nothing is touched)
+template <typename T>
+__global__ __launch_bounds__(256) void scale_by_scalar_kernel(T* __restrict__ x, const float* __restrict__ s, int64_t n8) {
+    const float sc = s[0];
+    if (sc == 1.0f) return;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+        float f[8];
+        Vec8<T>::load(x + i * 8, f);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) f[k] *= sc;
+        Vec8<T>::store(x + i * 8, f);
+    }
+}
+
+int ce_check(const char* name, const void* logits, int64_t rows, int64_t V, int64_t cut, int dtype) {
+    EZL_REQUIRE(dtype == 0 || dtype == 1, EZL_EUNSUPPORTED, "%s: dtype must be 0 (bf16) or 1 (fp32)", name);
+    EZL_REQUIRE(rows >= 0 && V > 0 && V % 8 == 0 && V < (1LL << 31), EZL_EUNSUPPORTED, "%s: vocab must be a multiple of 8", name);
+    EZL_REQUIRE(cut >= 0 && cut < V, EZL_EINVAL, "%s: bad cut_size", name);
+    EZL_REQUIRE(rows == 0 || logits, EZL_EINVAL, "%s: null logits", name);
+    EZL_REQUIRE(ezl_aligned16(logits), EZL_EINVAL, "%s: logits must be 16-byte aligned", name);
+    return EZL_OK;
+}
+
+inline unsigned ce_grid(int64_t rows) { return (unsigned)(rows < 256 * 8 ? (rows < 1 ? 1 : rows) : 256 * 8); }
+
+}  // namespace
+
+extern "C" int ezl_ce_prepare(const void* labels, const void* loss_mask, int mask_dtype, int64_t ignore_index, void* weights,
+                              void* count, int64_t n, void* stream) {
+    EZL_REQUIRE(n >= 0 && labels && weights && count, EZL_EINVAL, "ezl_ce_prepare: null pointer");
+    EZL_REQUIRE(mask_dtype >= 0 && mask_dtype <= 4 && (mask_dtype == 0 || loss_mask), EZL_EINVAL, "ezl_ce_prepare: bad loss_mask");
+    hipLaunchKernelGGL(ce_prepare_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const int64_t*)labels, loss_mask,
+                       mask_dtype, ignore_index, (float*)weights, (float*)count, n);
+    EZL_LAUNCH_CHECK("ezl_ce_prepare");
+    return EZL_OK;
+}
+
+extern "C" int ezl_ce_fwd(const void* logits, const void* labels, void* loss, void* lse, int64_t rows, int64_t vocab,
+                          int64_t cut_size, int dtype, void* stream) {
+    int rc = ce_check("ezl_ce_fwd", logits, rows, vocab, cut_size, dtype);
+    if (rc) return rc;
+    EZL_REQUIRE(rows == 0 || (labels && loss && lse), EZL_EINVAL, "ezl_ce_fwd: null pointer");
+    if (rows == 0) return EZL_OK;
+    const int V = (int)vocab, vend = (int)(vocab - cut_size);
+    const size_t row_bytes = (size_t)V * (dtype == 0 ? 2 : 4);
+    const bool in_lds = row_bytes <= 65536;
+    hipStream_t st = (hipStream_t)stream;
+#define LAUNCH(TT, L)                                                                                                  \
+    hipLaunchKernelGGL((ce_fwd_kernel<TT, L>), dim3(ce_grid(rows)), dim3(kCeBlock), (L) ? row_bytes : 0, st, (const TT*)logits, \
+                       (const int64_t*)labels, (float*)loss, (float*)lse, rows, V, vend)
+    if (dtype == 0) { if (in_lds) LAUNCH(bf16_t, true); else LAUNCH(bf16_t, false); }
+    else { if (in_lds) LAUNCH(float, true); else LAUNCH(float, false); }
+#undef LAUNCH
+    EZL_LAUNCH_CHECK("ezl_ce_fwd");
+    return EZL_OK;
+}
+
+extern "C" int ezl_ce_bwd(const void* logits, const void* labels, const void* lse, const void* grad_out, void* grad,
+                          int64_t rows, int64_t vocab, int64_t cut_size, int dtype, void* stream) {
+    int rc = ce_check("ezl_ce_bwd", logits, rows, vocab, cut_size, dtype);
+    if (rc) return rc;
+    EZL_REQUIRE(rows == 0 || (labels && lse && grad_out && grad), EZL_EINVAL, "ezl_ce_bwd: null pointer");
+    EZL_REQUIRE(ezl_aligned16(grad), EZL_EINVAL, "ezl_ce_bwd: grad must be 16-byte aligned");
+    if (rows == 0) return EZL_OK;
+    const int V = (int)vocab, vend = (int)(vocab - cut_size);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == 0)
+        hipLaunchKernelGGL((ce_bwd_kernel<bf16_t>), dim3(ce_grid(rows)), dim3(kCeBlock), 0, st, (const bf16_t*)logits,
+                           (const int64_t*)labels, (const float*)lse, (const float*)grad_out, (bf16_t*)grad, rows, V, vend);
+    else
+        hipLaunchKernelGGL((ce_bwd_kernel<float>), dim3(ce_grid(rows)), dim3(kCeBlock), 0, st, (const float*)logits,
+                           (const int64_t*)labels, (const float*)lse, (const float*)grad_out, (float*)grad, rows, V, vend);
+    EZL_LAUNCH_CHECK("ezl_ce_bwd");
+    return EZL_OK;
+}
+
+extern "C" int ezl_ce_fused(const void* logits, const void* labels, const void* weights, const void* count, void* loss_rows,
+                            void* grad, int64_t rows, int64_t vocab, int64_t cut_size, int dtype, void* stream) {
+    int rc = ce_check("ezl_ce_fused", logits, rows, vocab, cut_size, dtype);
+    if (rc) return rc;
+    EZL_REQUIRE(rows == 0 || (labels && weights && count && loss_rows && grad), EZL_EINVAL, "ezl_ce_fused: null pointer");
+    EZL_REQUIRE(ezl_aligned16(grad), EZL_EINVAL, "ezl_ce_fused: grad must be 16-byte aligned");
+    if (rows == 0) return EZL_OK;
+    const int V = (int)vocab, vend = (int)(vocab - cut_size);
+    const size_t row_bytes = (size_t)V * (dtype == 0 ? 2 : 4);
+    const bool in_lds = row_bytes <= 65536;
+    hipStream_t st = (hipStream_t)stream;
+#define LAUNCH(TT, L)                                                                                                    \
+    hipLaunchKernelGGL((ce_fused_kernel<TT, L>), dim3(ce_grid(rows)), dim3(kCeBlock), (L) ? row_bytes : 0, st, (const TT*)logits, \
+                       (const int64_t*)labels, (const float*)weights, (const float*)count, (float*)loss_rows, (TT*)grad, rows, \
+                       V, vend)
+    if (dtype == 0) { if (in_lds) LAUNCH(bf16_t, true); else LAUNCH(bf16_t, false); }
+    else { if (in_lds) LAUNCH(float, true); else LAUNCH(float, false); }
+#undef LAUNCH
+    EZL_LAUNCH_CHECK("ezl_ce_fused");
+    return EZL_OK;
+}
+
+extern "C" int ezl_ce_reduce(const void* loss_rows, const void* weights, const void* count, void* loss_out, int64_t n,
+                             void* stream) {
+    EZL_REQUIRE(n >= 0 && loss_rows && weights && count && loss_out, EZL_EINVAL, "ezl_ce_reduce: null pointer");
+    hipLaunchKernelGGL(ce_reduce_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const float*)loss_rows,
+                       (const float*)weights, (const float*)count, (float*)loss_out, n);
+    EZL_LAUNCH_CHECK("ezl_ce_reduce");
+    return EZL_OK;
+}
+
+extern "C" int ezl_scale_by_scalar(void* x, const void* scalar_f32, int64_t n, int dtype, void* stream) {
+    EZL_REQUIRE(dtype == 0 || dtype == 1, EZL_EUNSUPPORTED, "ezl_scale_by_scalar: dtype must be 0 (bf16) or 1 (fp32)");
+    EZL_REQUIRE(n >= 0 && n % 8 == 0 && (n == 0 || (x && scalar_f32)) && ezl_aligned16(x), EZL_EINVAL,
+                "ezl_scale_by_scalar: bad argument");
+    if (n == 0) return EZL_OK;
+    int64_t g = (n / 8 + 255) / 256;
+    if (g > 256 * 16) g = 256 * 16;
+    if (dtype == 0)
+        hipLaunchKernelGGL((scale_by_scalar_kernel<bf16_t>), dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, (bf16_t*)x,
+                           (const float*)scalar_f32, n / 8);
+    else
+        hipLaunchKernelGGL((scale_by_scalar_kernel<float>), dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, (float*)x,
+                           (const float*)scalar_f32, n / 8);
+    EZL_LAUNCH_CHECK("ezl_scale_by_scalar");
+    return EZL_OK;
+}

@@ -1,0 +1,320 @@
+// HBM-bound elementwise / gather kernels of the llama decoder-layer step (gfx950):
+// SwiGLU, rotary embedding, token-embedding gather / scatter-add, [b,s,h] <-> [s,b,h] row moves,
+// bf16 add and bf16 <-> fp32 casts.  All use 128-bit accesses (8 bf16 per lane).
+#include "common.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+
+inline unsigned grid_for(int64_t items, int per_block, int64_t cap = 256 * 32) {
+    int64_t g = (items + per_block - 1) / per_block;
+    if (g > cap) g = cap;
+    if (g < 1) g = 1;
+    return (unsigned)g;
+}
+
+__device__ __forceinline__ float sigmoidf_fast(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+// ---------------------------------------------------------------------------------------------
+// SwiGLU: out = silu(gate) * up     (llama/transformer.py:220-222, glu_activations.py:56-61)
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void swiglu_fwd_kernel(const bf16_t* __restrict__ gate, const bf16_t* __restrict__ up,
+                                                            bf16_t* __restrict__ out, int64_t n8) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += (int64_t)gridDim.x * kBlock) {
+        float g[8], u[8], o[8];
+        unpack8(ld_bf16x8(gate + i * 8), g);
+        unpack8(ld_bf16x8(up + i * 8), u);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) o[k] = g[k] * sigmoidf_fast(g[k]) * u[k];
+        st_bf16x8(out + i * 8, pack8(o));
+    }
+}
+
+// dgate = dout * up * s * (1 + g * (1 - s)),  dup = dout * g * s,  s = sigmoid(g)
+__global__ __launch_bounds__(kBlock) void swiglu_bwd_kernel(const bf16_t* __restrict__ dout, const bf16_t* __restrict__ gate,
+                                                            const bf16_t* __restrict__ up, bf16_t* __restrict__ dgate,
+                                                            bf16_t* __restrict__ dup, int64_t n8) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += (int64_t)gridDim.x * kBlock) {
+        float g[8], u[8], d[8], dg[8], du[8];
+        unpack8(ld_bf16x8(gate + i * 8), g);
+        unpack8(ld_bf16x8(up + i * 8), u);
+        unpack8(ld_bf16x8(dout + i * 8), d);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float s = sigmoidf_fast(g[k]);
+            dg[k] = d[k] * u[k] * s * (1.0f + g[k] * (1.0f - s));
+            du[k] = d[k] * g[k] * s;
+        }
+        st_bf16x8(dgate + i * 8, pack8(dg));
+        st_bf16x8(dup + i * 8, pack8(du));
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Rotary embedding (llama/positional_embeddings.py:17-36, 94-96, 105-122)
+// ---------------------------------------------------------------------------------------------
+// cos/sin table [npos, d/2] in fp32: theta = (p / scale_factor) * inv_freq[j]  (:21-23)
+__global__ __launch_bounds__(kBlock) void rope_table_kernel(const float* __restrict__ inv_freq, float* __restrict__ cosb,
+                                                            float* __restrict__ sinb, int64_t npos, int half,
+                                                            float scale_factor) {
+    const int64_t n = npos * half;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t p = i / half;
+        const int j = (int)(i % half);
+        const float t = (float)p / scale_factor;
+        const float th = t * inv_freq[j];
+        cosb[i] = cosf(th);
+        sinb[i] = sinf(th);
+    }
+}
+
+// x [rows = s*b (s-major), nheads, d] with a row stride; one work item = 8 low-half + 8 high-half
+// elements of one head.  out1 = x1*c - sign*x2*s ; out2 = x2*c + sign*x1*s  (sign = -1: backward).
+__global__ __launch_bounds__(kBlock) void rope_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ out,
+                                                      const float* __restrict__ cosb, const float* __restrict__ sinb,
+                                                      const int64_t* __restrict__ position_ids, int64_t rows, int s,
+                                                      int b, int nheads, int d, int64_t in_stride, int64_t out_stride,
+                                                      int64_t npos, float sign) {
+    const int half = d >> 1;
+    const int per_head = half >> 3;
+    const int64_t items = rows * nheads * per_head;
+    for (int64_t it = (int64_t)blockIdx.x * kBlock + threadIdx.x; it < items; it += (int64_t)gridDim.x * kBlock) {
+        const int j8 = (int)(it % per_head);
+        const int64_t rh = it / per_head;
+        const int head = (int)(rh % nheads);
+        const int64_t row = rh / nheads;
+        const int si = (int)(row / b), bi = (int)(row % b);
+        int64_t pos = position_ids ? position_ids[(int64_t)bi * s + si] : si;
+        pos = pos < 0 ? 0 : (pos >= npos ? npos - 1 : pos);
+        const float* cp = cosb + pos * half + j8 * 8;
+        const float* sp = sinb + pos * half + j8 * 8;
+        const bf16_t* xi = x + row * in_stride + (int64_t)head * d + j8 * 8;
+        bf16_t* xo = out + row * out_stride + (int64_t)head * d + j8 * 8;
+        float a[8], c[8], o1[8], o2[8];
+        unpack8(ld_bf16x8(xi), a);
+        unpack8(ld_bf16x8(xi + half), c);
+        const f32x4 c0 = *reinterpret_cast<const f32x4*>(cp), c1 = *reinterpret_cast<const f32x4*>(cp + 4);
+        const f32x4 s0 = *reinterpret_cast<const f32x4*>(sp), s1 = *reinterpret_cast<const f32x4*>(sp + 4);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float cs = k < 4 ? c0[k] : c1[k - 4];
+            const float sn = sign * (k < 4 ? s0[k] : s1[k - 4]);
+            o1[k] = a[k] * cs - c[k] * sn;
+            o2[k] = c[k] * cs + a[k] * sn;
+        }
+        st_bf16x8(xo, pack8(o1));
+        st_bf16x8(xo + half, pack8(o2));
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Token embedding (base_modules/layers/vocab_parallel_emb.py:106-137, TP=1)
+// ---------------------------------------------------------------------------------------------
+// out[r, :] = W[ids[r], :]; an id outside [0, V) raises the flag and yields a zero row.
+__global__ __launch_bounds__(kBlock) void embed_gather_kernel(const int64_t* __restrict__ ids, const bf16_t* __restrict__ W,
+                                                              bf16_t* __restrict__ out, int64_t rows, int h, int64_t V,
+                                                              int* __restrict__ bad_flag) {
+    const int h8 = h >> 3;
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+        const int64_t id = ids[r];
+        const bool ok = id >= 0 && id < V;
+        if (!ok && threadIdx.x == 0) atomicOr(bad_flag, id >= V ? 1 : 2);
+        for (int c = threadIdx.x; c < h8; c += kBlock) {
+            bf16x8 v;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[k] = (bf16_t)0.0f;
+            if (ok) v = ld_bf16x8(W + id * h + c * 8);
+            st_bf16x8(out + r * h + c * 8, v);
+        }
+    }
+}
+
+// dW[ids[r], :] += dY[r, :] in fp32 (hardware float atomics: summation order is not fixed)
+__global__ __launch_bounds__(kBlock) void embed_scatter_add_kernel(const int64_t* __restrict__ ids,
+                                                                   const bf16_t* __restrict__ dY, float* __restrict__ dW,
+                                                                   int64_t rows, int h, int64_t V) {
+    const int h8 = h >> 3;
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+        const int64_t id = ids[r];
+        if (id < 0 || id >= V) continue;
+        for (int c = threadIdx.x; c < h8; c += kBlock) {
+            float g[8];
+            unpack8(ld_bf16x8(dY + r * h + c * 8), g);
+            float* dst = dW + id * h + c * 8;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) atomicAdd(dst + k, g[k]);
+        }
+    }
+}
+
+// y[j, i, :] = x[i, j, :]  for x [d0, d1, inner]   (llama/llama.py:157-168,175-179)
+__global__ __launch_bounds__(kBlock) void transpose01_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ y, int64_t d0,
+                                                             int64_t d1, int inner) {
+    const int i8 = inner >> 3;
+    const int64_t rows = d0 * d1;
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+        const int64_t i = r / d1, j = r % d1;
+        const bf16_t* src = x + r * inner;
+        bf16_t* dst = y + (j * d0 + i) * inner;
+        for (int c = threadIdx.x; c < i8; c += kBlock) st_bf16x8(dst + c * 8, ld_bf16x8(src + c * 8));
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void add_kernel(const bf16_t* __restrict__ a, const bf16_t* __restrict__ b,
+                                                     bf16_t* __restrict__ out, int64_t n8) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += (int64_t)gridDim.x * kBlock) {
+        float x[8], y[8];
+        unpack8(ld_bf16x8(a + i * 8), x);
+        unpack8(ld_bf16x8(b + i * 8), y);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) x[k] += y[k];
+        st_bf16x8(out + i * 8, pack8(x));
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void bf16_to_f32_kernel(const bf16_t* __restrict__ in, float* __restrict__ out, int64_t n8) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += (int64_t)gridDim.x * kBlock) {
+        float x[8];
+        unpack8(ld_bf16x8(in + i * 8), x);
+        f32x4 lo = {x[0], x[1], x[2], x[3]}, hi = {x[4], x[5], x[6], x[7]};
+        *reinterpret_cast<f32x4*>(out + i * 8) = lo;
+        *reinterpret_cast<f32x4*>(out + i * 8 + 4) = hi;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void f32_to_bf16_kernel(const float* __restrict__ in, bf16_t* __restrict__ out, int64_t n8) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += (int64_t)gridDim.x * kBlock) {
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(in + i * 8), hi = *reinterpret_cast<const f32x4*>(in + i * 8 + 4);
+        float x[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        st_bf16x8(out + i * 8, pack8(x));
+    }
+}
+
+}  // namespace
+
+extern "C" int ezl_swiglu_fwd(const void* gate, const void* up, void* out, int64_t n, void* stream) {
+    EZL_REQUIRE(n >= 0 && n % 8 == 0, EZL_EUNSUPPORTED, "ezl_swiglu_fwd: n must be a multiple of 8");
+    EZL_REQUIRE(ezl_aligned16(gate) && ezl_aligned16(up) && ezl_aligned16(out) && (n == 0 || (gate && up && out)), EZL_EINVAL,
+                "ezl_swiglu_fwd: null or misaligned pointer");
+    if (n == 0) return EZL_OK;
+    hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(grid_for(n / 8, kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
+                       (const bf16_t*)gate, (const bf16_t*)up, (bf16_t*)out, n / 8);
+    EZL_LAUNCH_CHECK("ezl_swiglu_fwd");
+    return EZL_OK;
+}
+
+extern "C" int ezl_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate, void* dup, int64_t n,
+                              void* stream) {
+    EZL_REQUIRE(n >= 0 && n % 8 == 0, EZL_EUNSUPPORTED, "ezl_swiglu_bwd: n must be a multiple of 8");
+    EZL_REQUIRE(ezl_aligned16(dout) && ezl_aligned16(gate) && ezl_aligned16(up) && ezl_aligned16(dgate) && ezl_aligned16(dup) &&
+                    (n == 0 || (dout && gate && up && dgate && dup)),
+                EZL_EINVAL, "ezl_swiglu_bwd: null or misaligned pointer");
+    if (n == 0) return EZL_OK;
+    hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(grid_for(n / 8, kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
+                       (const bf16_t*)dout, (const bf16_t*)gate, (const bf16_t*)up, (bf16_t*)dgate, (bf16_t*)dup, n / 8);
+    EZL_LAUNCH_CHECK("ezl_swiglu_bwd");
+    return EZL_OK;
+}
+
+extern "C" int ezl_rope_table(const void* inv_freq, void* cos_out, void* sin_out, int64_t npos, int64_t half_dim,
+                              float scale_factor, void* stream) {
+    EZL_REQUIRE(npos > 0 && half_dim > 0 && scale_factor > 0.f && inv_freq && cos_out && sin_out, EZL_EINVAL,
+                "ezl_rope_table: bad argument");
+    hipLaunchKernelGGL(rope_table_kernel, dim3(grid_for(npos * half_dim, kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
+                       (const float*)inv_freq, (float*)cos_out, (float*)sin_out, npos, (int)half_dim, scale_factor);
+    EZL_LAUNCH_CHECK("ezl_rope_table");
+    return EZL_OK;
+}
+
+extern "C" int ezl_rope_apply(const void* x, void* out, const void* cos_table, const void* sin_table,
+                              const void* position_ids, int64_t s, int64_t b, int64_t nheads, int64_t d,
+                              int64_t in_row_stride, int64_t out_row_stride, int64_t npos, int backward, void* stream) {
+    EZL_REQUIRE(s >= 0 && b > 0 && nheads > 0 && d > 0 && d % 16 == 0, EZL_EUNSUPPORTED,
+                "ezl_rope_apply: head dim must be a multiple of 16 (got %lld)", (long long)d);
+    EZL_REQUIRE(in_row_stride % 8 == 0 && out_row_stride % 8 == 0 && in_row_stride >= nheads * d && out_row_stride >= nheads * d,
+                EZL_EINVAL, "ezl_rope_apply: bad row stride");
+    EZL_REQUIRE(npos >= 1 && (position_ids || npos >= s), EZL_EINVAL, "ezl_rope_apply: cos/sin table shorter than the sequence");
+    EZL_REQUIRE(x && out && cos_table && sin_table && ezl_aligned16(x) && ezl_aligned16(out) && ezl_aligned16(cos_table) &&
+                    ezl_aligned16(sin_table),
+                EZL_EINVAL, "ezl_rope_apply: null or misaligned pointer");
+    EZL_REQUIRE(s < (1LL << 31) && b < (1LL << 31), EZL_EUNSUPPORTED, "ezl_rope_apply: shape too large");
+    if (s == 0) return EZL_OK;
+    const int64_t items = s * b * nheads * (d / 16);
+    hipLaunchKernelGGL(rope_kernel, dim3(grid_for(items, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, (const bf16_t*)x,
+                       (bf16_t*)out, (const float*)cos_table, (const float*)sin_table, (const int64_t*)position_ids, s * b,
+                       (int)s, (int)b, (int)nheads, (int)d, in_row_stride, out_row_stride, npos, backward ? -1.0f : 1.0f);
+    EZL_LAUNCH_CHECK("ezl_rope_apply");
+    return EZL_OK;
+}
+
+extern "C" int ezl_embed_gather(const void* ids, const void* weight, void* out, void* bad_flag, int64_t rows, int64_t h,
+                                int64_t vocab, void* stream) {
+    EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h < (1LL << 31) && vocab > 0, EZL_EUNSUPPORTED,
+                "ezl_embed_gather: h must be a multiple of 8");
+    EZL_REQUIRE(bad_flag && (rows == 0 || (ids && weight && out)) && ezl_aligned16(weight) && ezl_aligned16(out), EZL_EINVAL,
+                "ezl_embed_gather: null or misaligned pointer");
+    if (rows == 0) return EZL_OK;
+    hipLaunchKernelGGL(embed_gather_kernel, dim3(grid_for(rows, 1)), dim3(kBlock), 0, (hipStream_t)stream, (const int64_t*)ids,
+                       (const bf16_t*)weight, (bf16_t*)out, rows, (int)h, vocab, (int*)bad_flag);
+    EZL_LAUNCH_CHECK("ezl_embed_gather");
+    return EZL_OK;
+}
+
+extern "C" int ezl_embed_scatter_add(const void* ids, const void* dy, void* dweight_f32, int64_t rows, int64_t h,
+                                     int64_t vocab, void* stream) {
+    EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h < (1LL << 31) && vocab > 0, EZL_EUNSUPPORTED,
+                "ezl_embed_scatter_add: h must be a multiple of 8");
+    EZL_REQUIRE((rows == 0 || (ids && dy && dweight_f32)) && ezl_aligned16(dy), EZL_EINVAL,
+                "ezl_embed_scatter_add: null or misaligned pointer");
+    if (rows == 0) return EZL_OK;
+    hipLaunchKernelGGL(embed_scatter_add_kernel, dim3(grid_for(rows, 1)), dim3(kBlock), 0, (hipStream_t)stream,
+                       (const int64_t*)ids, (const bf16_t*)dy, (float*)dweight_f32, rows, (int)h, vocab);
+    EZL_LAUNCH_CHECK("ezl_embed_scatter_add");
+    return EZL_OK;
+}
+
+extern "C" int ezl_transpose01(const void* x, void* y, int64_t d0, int64_t d1, int64_t inner, void* stream) {
+    EZL_REQUIRE(d0 >= 0 && d1 >= 0 && inner > 0 && inner % 8 == 0 && inner < (1LL << 31), EZL_EUNSUPPORTED,
+                "ezl_transpose01: inner must be a multiple of 8");
+    EZL_REQUIRE((d0 * d1 == 0 || (x && y)) && ezl_aligned16(x) && ezl_aligned16(y), EZL_EINVAL,
+                "ezl_transpose01: null or misaligned pointer");
+    if (d0 * d1 == 0) return EZL_OK;
+    hipLaunchKernelGGL(transpose01_kernel, dim3(grid_for(d0 * d1, 1)), dim3(kBlock), 0, (hipStream_t)stream, (const bf16_t*)x,
+                       (bf16_t*)y, d0, d1, (int)inner);
+    EZL_LAUNCH_CHECK("ezl_transpose01");
+    return EZL_OK;
+}
+
+extern "C" int ezl_add(const void* a, const void* b, void* out, int64_t n, void* stream) {
+    EZL_REQUIRE(n >= 0 && n % 8 == 0, EZL_EUNSUPPORTED, "ezl_add: n must be a multiple of 8");
+    EZL_REQUIRE((n == 0 || (a && b && out)) && ezl_aligned16(a) && ezl_aligned16(b) && ezl_aligned16(out), EZL_EINVAL,
+                "ezl_add: null or misaligned pointer");
+    if (n == 0) return EZL_OK;
+    hipLaunchKernelGGL(add_kernel, dim3(grid_for(n / 8, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, (const bf16_t*)a,
+                       (const bf16_t*)b, (bf16_t*)out, n / 8);
+    EZL_LAUNCH_CHECK("ezl_add");
+    return EZL_OK;
+}
+
+extern "C" int ezl_cast_bf16_to_f32(const void* in, void* out, int64_t n, void* stream) {
+    EZL_REQUIRE(n >= 0 && n % 8 == 0, EZL_EUNSUPPORTED, "ezl_cast_bf16_to_f32: n must be a multiple of 8");
+    EZL_REQUIRE((n == 0 || (in && out)) && ezl_aligned16(in) && ezl_aligned16(out), EZL_EINVAL,
+                "ezl_cast_bf16_to_f32: null or misaligned pointer");
+    if (n == 0) return EZL_OK;
+    hipLaunchKernelGGL(bf16_to_f32_kernel, dim3(grid_for(n / 8, kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
+                       (const bf16_t*)in, (float*)out, n / 8);
+    EZL_LAUNCH_CHECK("ezl_cast_bf16_to_f32");
+    return EZL_OK;
+}
+
+extern "C" int ezl_cast_f32_to_bf16(const void* in, void* out, int64_t n, void* stream) {
+    EZL_REQUIRE(n >= 0 && n % 8 == 0, EZL_EUNSUPPORTED, "ezl_cast_f32_to_bf16: n must be a multiple of 8");
+    EZL_REQUIRE((n == 0 || (in && out)) && ezl_aligned16(in) && ezl_aligned16(out), EZL_EINVAL,
+                "ezl_cast_f32_to_bf16: null or misaligned pointer");
+    if (n == 0) return EZL_OK;
+    hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(grid_for(n / 8, kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
+                       (const float*)in, (bf16_t*)out, n / 8);
+    EZL_LAUNCH_CHECK("ezl_cast_f32_to_bf16");
+    return EZL_OK;
+}

@@ -1,0 +1,273 @@
+// RMSNorm forward / backward for gfx950 (HBM-bound).
+//
+// Restates base_modules/layers/fused_layer_norm.py:49-71 of the reference (the fp32-accumulate
+// form its fused path uses): y = x * rsqrt(mean(x^2) + eps) * w, with the optional residual add
+// of llama/transformer.py:786 fused in front (sum rounded to bf16 first, as the reference's bf16
+// tensor add does).
+//
+// Layout: rows of h bf16, h % 8 == 0, h <= 8192.  A row is owned by TPR = min(256, h/8 rounded up
+// to a wave) threads, each holding NCHUNK 128-bit column groups in registers, so a row is read
+// from HBM exactly once.  Row sums reduce with wave shuffles, then across the (<= 4) waves of the
+// row slot through a double-buffered LDS cell (one barrier per row).
+#include "common.h"
+
+namespace {
+
+template <int NCHUNK, bool HAS_RES>
+__global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ res,
+                                                          const bf16_t* __restrict__ w, bf16_t* __restrict__ y,
+                                                          bf16_t* __restrict__ sum_out, float* __restrict__ rstd_out,
+                                                          int T, int h, float eps, int tpr) {
+    __shared__ float red[2][4][4];  // [parity][row slot][wave in slot]
+    const int rpb = 256 / tpr;             // row slots per block
+    const int slot = threadIdx.x / tpr;    // which row slot
+    const int tin = threadIdx.x % tpr;     // thread within the row
+    const int wis = tin >> 6;              // wave within the slot
+    const int nws = tpr >> 6;              // waves per slot
+    const int lane = threadIdx.x & 63;
+    float wv[NCHUNK][8];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+        const int col = (c * tpr + tin) * 8;
+        if (col < h) unpack8(ld_bf16x8(w + col), wv[c]);
+    }
+    int parity = 0;
+    // every thread of the block runs the same number of iterations (barrier inside)
+    for (int row0 = blockIdx.x * rpb; row0 < T; row0 += gridDim.x * rpb) {
+        const int row = row0 + slot;
+        const bool live = row < T;
+        const size_t base = (size_t)row * h;
+        float xv[NCHUNK][8];
+        float ss = 0.f;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            const int col = (c * tpr + tin) * 8;
+            if (live && col < h) {
+                unpack8(ld_bf16x8(x + base + col), xv[c]);
+                if (HAS_RES) {
+                    float r[8];
+                    unpack8(ld_bf16x8(res + base + col), r);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) xv[c][i] = (float)(bf16_t)(xv[c][i] + r[i]);
+                    st_bf16x8(sum_out + base + col, pack8(xv[c]));
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) ss += xv[c][i] * xv[c][i];
+            }
+        }
+        ss = wave_sum(ss);
+        if (nws > 1) {
+            if (lane == 0) red[parity][slot][wis] = ss;
+            __syncthreads();
+            ss = 0.f;
+            for (int i = 0; i < nws; ++i) ss += red[parity][slot][i];
+            parity ^= 1;
+        }
+        const float rs = rsqrtf(ss / (float)h + eps);
+        if (live && tin == 0) rstd_out[row] = rs;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            const int col = (c * tpr + tin) * 8;
+            if (live && col < h) {
+                float o[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) o[i] = xv[c][i] * rs * wv[c][i];
+                st_bf16x8(y + base + col, pack8(o));
+            }
+        }
+    }
+}
+
+// dx = rstd * (g - xhat * mean(g * xhat)),  g = dy * w, xhat = x * rstd;  dw = sum_rows dy * xhat.
+// Each thread keeps the dw partial of its own columns over all rows the block visits; the row slots
+// of a block are then folded through LDS and one partial row per block goes to HBM.
+template <int NCHUNK, bool HAS_DRES>
+__global__ __launch_bounds__(1024) void rmsnorm_bwd_kernel(const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
+                                                           const bf16_t* __restrict__ w, const float* __restrict__ rstd,
+                                                           const bf16_t* __restrict__ dres, bf16_t* __restrict__ dx,
+                                                           float* __restrict__ dw_partial, int T, int h, int tpr) {
+    extern __shared__ float fold[];  // h floats
+    __shared__ float red[2][16][4];
+    const int rpb = 1024 / tpr;
+    const int slot = threadIdx.x / tpr;
+    const int tin = threadIdx.x % tpr;
+    const int wis = tin >> 6;
+    const int nws = tpr >> 6;
+    const int lane = threadIdx.x & 63;
+    float wv[NCHUNK][8];
+    float dwacc[NCHUNK][8];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+        const int col = (c * tpr + tin) * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { dwacc[c][i] = 0.f; wv[c][i] = 0.f; }
+        if (col < h) unpack8(ld_bf16x8(w + col), wv[c]);
+    }
+    int parity = 0;
+    const float inv_h = 1.0f / (float)h;
+    for (int row0 = blockIdx.x * rpb; row0 < T; row0 += gridDim.x * rpb) {
+        const int row = row0 + slot;
+        const bool live = row < T;
+        const size_t base = (size_t)row * h;
+        const float rs = live ? rstd[row] : 0.f;
+        bf16x8 xr[NCHUNK], dyr[NCHUNK];
+        float dot = 0.f;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            const int col = (c * tpr + tin) * 8;
+            if (live && col < h) {
+                xr[c] = ld_bf16x8(x + base + col);
+                dyr[c] = ld_bf16x8(dy + base + col);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) dot += (float)dyr[c][i] * wv[c][i] * ((float)xr[c][i] * rs);
+            }
+        }
+        dot = wave_sum(dot);
+        if (nws > 1) {
+            if (lane == 0) red[parity][slot][wis] = dot;
+            __syncthreads();
+            dot = 0.f;
+            for (int i = 0; i < nws; ++i) dot += red[parity][slot][i];
+            parity ^= 1;
+        }
+        const float cmean = dot * inv_h;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            const int col = (c * tpr + tin) * 8;
+            if (live && col < h) {
+                float o[8];
+                float dr[8];
+                if (HAS_DRES) unpack8(ld_bf16x8(dres + base + col), dr);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float xhat = (float)xr[c][i] * rs;
+                    const float dyv = (float)dyr[c][i];
+                    o[i] = rs * (dyv * wv[c][i] - xhat * cmean);
+                    if (HAS_DRES) o[i] += dr[i];
+                    dwacc[c][i] += dyv * xhat;
+                }
+                st_bf16x8(dx + base + col, pack8(o));
+            }
+        }
+    }
+    // fold the row slots of this block: slot 0 stores, the others add, one barrier per slot
+    for (int s = 0; s < rpb; ++s) {
+        if (slot == s) {
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c) {
+                const int col = (c * tpr + tin) * 8;
+                if (col < h) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        if (s == 0) fold[col + i] = dwacc[c][i];
+                        else fold[col + i] += dwacc[c][i];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    for (int j = threadIdx.x; j < h; j += 1024) dw_partial[(size_t)blockIdx.x * h + j] = fold[j];
+}
+
+// out[col] (+)= sum_r partial[r][col];  64 columns per block, 4 row groups folded through LDS.
+__global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ partial, int nrows, int ncols,
+                                                     bf16_t* __restrict__ out_bf16, float* __restrict__ out_f32,
+                                                     int accumulate) {
+    __shared__ float s[4][64];
+    const int c = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int col = blockIdx.x * 64 + c;
+    float acc = 0.f;
+    if (col < ncols)
+        for (int r = g; r < nrows; r += 4) acc += partial[(size_t)r * ncols + col];
+    s[g][c] = acc;
+    __syncthreads();
+    if (g == 0 && col < ncols) {
+        const float v = s[0][c] + s[1][c] + s[2][c] + s[3][c];
+        if (out_f32) out_f32[col] = accumulate ? out_f32[col] + v : v;
+        else out_bf16[col] = (bf16_t)v;
+    }
+}
+
+int tpr_for(int h) {
+    int t = (h / 8 + 63) / 64 * 64;
+    return t < 64 ? 64 : (t > 256 ? 256 : t);
+}
+
+}  // namespace
+
+extern "C" int ezl_rmsnorm_fwd(const void* x, const void* residual, const void* weight, void* y, void* sum_out,
+                               void* rstd, int64_t rows, int64_t h, float eps, void* stream) {
+    EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h <= 8192, EZL_EUNSUPPORTED,
+                "ezl_rmsnorm_fwd: need h %% 8 == 0 and h <= 8192 (got h=%lld)", (long long)h);
+    EZL_REQUIRE(x && weight && y && rstd, EZL_EINVAL, "ezl_rmsnorm_fwd: null pointer");
+    EZL_REQUIRE((residual == nullptr) == (sum_out == nullptr), EZL_EINVAL,
+                "ezl_rmsnorm_fwd: residual and sum_out go together");
+    EZL_REQUIRE(ezl_aligned16(x) && ezl_aligned16(weight) && ezl_aligned16(y) && ezl_aligned16(residual) &&
+                    ezl_aligned16(sum_out),
+                EZL_EINVAL, "ezl_rmsnorm_fwd: pointers must be 16-byte aligned");
+    if (rows == 0) return EZL_OK;
+    const int tpr = tpr_for((int)h);
+    const int nchunk = ((int)h + tpr * 8 - 1) / (tpr * 8);
+    const int rpb = 256 / tpr;
+    int64_t grid = (rows + rpb - 1) / rpb;
+    if (grid > 256 * 16) grid = 256 * 16;
+    hipStream_t st = (hipStream_t)stream;
+#define LAUNCH(NC, RES)                                                                                             \
+    hipLaunchKernelGGL((rmsnorm_fwd_kernel<NC, RES>), dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)x,      \
+                       (const bf16_t*)residual, (const bf16_t*)weight, (bf16_t*)y, (bf16_t*)sum_out, (float*)rstd, \
+                       (int)rows, (int)h, eps, tpr)
+    EZL_REQUIRE(rows < (1LL << 31), EZL_EUNSUPPORTED, "ezl_rmsnorm_fwd: too many rows");
+    if (residual) {
+        if (nchunk == 1) LAUNCH(1, true); else if (nchunk == 2) LAUNCH(2, true); else LAUNCH(4, true);
+    } else {
+        if (nchunk == 1) LAUNCH(1, false); else if (nchunk == 2) LAUNCH(2, false); else LAUNCH(4, false);
+    }
+#undef LAUNCH
+    EZL_LAUNCH_CHECK("ezl_rmsnorm_fwd");
+    return EZL_OK;
+}
+
+extern "C" int64_t ezl_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t h) {
+    (void)rows;
+    return (int64_t)256 * h * (int64_t)sizeof(float);
+}
+
+extern "C" int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const void* rstd,
+                               const void* dresidual, void* dx, void* dw_bf16, void* dw_f32, int accumulate,
+                               void* workspace, int64_t workspace_bytes, int64_t rows, int64_t h, void* stream) {
+    EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h <= 8192, EZL_EUNSUPPORTED,
+                "ezl_rmsnorm_bwd: need h %% 8 == 0 and h <= 8192 (got h=%lld)", (long long)h);
+    EZL_REQUIRE(dy && x && weight && rstd && dx && workspace, EZL_EINVAL, "ezl_rmsnorm_bwd: null pointer");
+    EZL_REQUIRE((dw_bf16 != nullptr) != (dw_f32 != nullptr), EZL_EINVAL,
+                "ezl_rmsnorm_bwd: exactly one of dw_bf16 / dw_f32");
+    EZL_REQUIRE(workspace_bytes >= ezl_rmsnorm_bwd_workspace_bytes(rows, h), EZL_EINVAL,
+                "ezl_rmsnorm_bwd: workspace too small");
+    EZL_REQUIRE(ezl_aligned16(dy) && ezl_aligned16(x) && ezl_aligned16(weight) && ezl_aligned16(dx) &&
+                    ezl_aligned16(dresidual),
+                EZL_EINVAL, "ezl_rmsnorm_bwd: pointers must be 16-byte aligned");
+    EZL_REQUIRE(rows < (1LL << 31), EZL_EUNSUPPORTED, "ezl_rmsnorm_bwd: too many rows");
+    hipStream_t st = (hipStream_t)stream;
+    const int tpr = tpr_for((int)h);
+    const int nchunk = ((int)h + tpr * 8 - 1) / (tpr * 8);
+    const int rpb = 1024 / tpr;
+    int64_t grid = (rows + rpb - 1) / rpb;
+    if (grid > 256) grid = 256;
+    if (grid < 1) grid = 1;  // rows == 0 still produces a zero dw
+    const size_t smem = (size_t)h * sizeof(float);
+#define LAUNCH(NC, DR)                                                                                            \
+    hipLaunchKernelGGL((rmsnorm_bwd_kernel<NC, DR>), dim3((unsigned)grid), dim3(1024), smem, st, (const bf16_t*)dy, \
+                       (const bf16_t*)x, (const bf16_t*)weight, (const float*)rstd, (const bf16_t*)dresidual,     \
+                       (bf16_t*)dx, (float*)workspace, (int)rows, (int)h, tpr)
+    if (dresidual) {
+        if (nchunk == 1) LAUNCH(1, true); else if (nchunk == 2) LAUNCH(2, true); else LAUNCH(4, true);
+    } else {
+        if (nchunk == 1) LAUNCH(1, false); else if (nchunk == 2) LAUNCH(2, false); else LAUNCH(4, false);
+    }
+#undef LAUNCH
+    EZL_LAUNCH_CHECK("ezl_rmsnorm_bwd");
+    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((h + 63) / 64)), dim3(256), 0, st, (const float*)workspace,
+                       (int)grid, (int)h, (bf16_t*)dw_bf16, (float*)dw_f32, accumulate);
+    EZL_LAUNCH_CHECK("ezl_rmsnorm_bwd(colsum)");
+    return EZL_OK;
+}

@@ -1,0 +1,118 @@
+/* C ABI of libezl: gfx950 kernels for the llama decoder-layer training step at TP=1.
+ *
+ * The reference (ModelTC/EasyLLM) has no FFI of its own for this path: its GPU kernels are reached
+ * through optional Python imports (flash-attn, dropout_layer_norm, torch.matmul).  Each entry point
+ * below names the reference call it stands in for (paths relative to the reference tree).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated otherwise; buffers are owned by the caller;
+ *     nothing here allocates or frees device memory; workspaces are passed in;
+ *   - bf16 tensors: base 16-byte aligned, innermost dimension contiguous and a multiple of 8;
+ *   - `stream` is a hipStream_t (NULL = default stream); all work is enqueued there, no host sync;
+ *   - return 0 on success, a negative EZL_E* code otherwise; ezl_last_error() returns the message
+ *     of the last failure on the calling thread;
+ *   - re-entrant: no global mutable state; callable from any host thread (autograd workers included).
+ */
+#ifndef EZL_H
+#define EZL_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EZL_OK 0
+#define EZL_EINVAL (-1)       /* bad pointer / size / alignment */
+#define EZL_EUNSUPPORTED (-2) /* shape or dtype outside what the kernels cover */
+#define EZL_EHIP (-3)         /* the HIP runtime refused the launch */
+
+int ezl_version(void);
+const char* ezl_last_error(void);
+
+/* ---- RMSNorm: base_modules/layers/fused_layer_norm.py:49-71 (flash_attn rms_norm seam :56-57) ----
+ * y = (x [+ residual]) * rsqrt(mean(.^2) + eps) * weight, rows of h bf16 (h % 8 == 0, h <= 8192).
+ * residual/sum_out are both NULL or both given (the residual add of llama/transformer.py:786 fused
+ * in; sum_out receives x + residual rounded to bf16).  rstd: fp32 [rows], kept for backward. */
+int ezl_rmsnorm_fwd(const void* x, const void* residual, const void* weight, void* y, void* sum_out, void* rstd,
+                    int64_t rows, int64_t h, float eps, void* stream);
+int64_t ezl_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t h);
+/* dx = d/dx of the above (+ dresidual if given); dw goes to exactly one of dw_bf16 [h] (overwritten)
+ * or dw_f32 [h] (overwritten, or added to when accumulate != 0). */
+int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const void* rstd, const void* dresidual, void* dx,
+                    void* dw_bf16, void* dw_f32, int accumulate, void* workspace, int64_t workspace_bytes, int64_t rows,
+                    int64_t h, void* stream);
+
+/* ---- SwiGLU: llama/transformer.py:220-222 + base_modules/layers/glu_activations.py:56-61 ---- */
+int ezl_swiglu_fwd(const void* gate, const void* up, void* out, int64_t n, void* stream);
+int ezl_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate, void* dup, int64_t n, void* stream);
+
+/* ---- rotary embedding: llama/positional_embeddings.py:17-36 (table), :94-96,105-122 (apply) ----
+ * table: cos/sin fp32 [npos, half_dim], theta = (p / scale_factor) * inv_freq[j].
+ * apply: x/out bf16 [s*b rows (s-major), nheads, d] with row strides in elements (out may alias x);
+ * position_ids int64 [b, s] or NULL (position = s index); backward != 0 rotates by -theta. */
+int ezl_rope_table(const void* inv_freq, void* cos_out, void* sin_out, int64_t npos, int64_t half_dim, float scale_factor,
+                   void* stream);
+int ezl_rope_apply(const void* x, void* out, const void* cos_table, const void* sin_table, const void* position_ids, int64_t s,
+                   int64_t b, int64_t nheads, int64_t d, int64_t in_row_stride, int64_t out_row_stride, int64_t npos,
+                   int backward, void* stream);
+
+/* ---- token embedding: base_modules/layers/vocab_parallel_emb.py:106-137 (F.embedding, TP=1) ----
+ * gather: out[r] = weight[ids[r]] (bit-exact row copy); an id outside [0, vocab) ORs 1 (id >= vocab)
+ * or 2 (id < 0) into *bad_flag (device int32) and yields a zero row.
+ * scatter_add: dweight_f32[ids[r]] += dy[r] with fp32 atomics (summation order not fixed). */
+int ezl_embed_gather(const void* ids, const void* weight, void* out, void* bad_flag, int64_t rows, int64_t h, int64_t vocab,
+                     void* stream);
+int ezl_embed_scatter_add(const void* ids, const void* dy, void* dweight_f32, int64_t rows, int64_t h, int64_t vocab,
+                          void* stream);
+
+/* ---- layout / dtype plumbing of llama/llama.py:145-188 (transpose, undo, float16_to_fp32) ---- */
+int ezl_transpose01(const void* x, void* y, int64_t d0, int64_t d1, int64_t inner, void* stream); /* y[j,i,:] = x[i,j,:] */
+int ezl_add(const void* a, const void* b, void* out, int64_t n, void* stream); /* residual add, transformer.py:797 */
+int ezl_cast_bf16_to_f32(const void* in, void* out, int64_t n, void* stream);
+int ezl_cast_f32_to_bf16(const void* in, void* out, int64_t n, void* stream);
+
+/* ---- linear layers: column_parallel_linear.py:42 (fwd), :68 (dgrad), :99 (wgrad);
+ *      row_parallel_linear.py:113; llama/lm_head.py:62 ----
+ * C[M,N] (=|+=) A * B, bf16 operands, fp32 accumulation.
+ *   A: a_kc ? A[m*lda + k] : A[k*lda + m]     B: b_kc ? B[n*ldb + k] : B[k*ldb + n]
+ * out_dtype 0 = bf16, 1 = fp32. */
+int ezl_gemm_bf16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                  int a_kc, int b_kc, int out_dtype, int accumulate, void* stream);
+
+/* ---- attention: FlashAttention.forward, llama/transformer.py:83-143 (flash_attn_varlen_* seams
+ *      :106-115) ----
+ * q [T, nq, d], k/v [T, nk, d] bf16, d in {64, 128}; token n lives at
+ * (n / s_len) * batch_stride + (n % s_len) * seq_stride (elements) + head * d.
+ * cu_seqlens: int32 [ndocs + 1] or NULL (documents = the T / s_len batch rows; pass ndocs = T / s_len).
+ * lse / delta: fp32 [nq, T].  strides (HOST pointer): fwd 8 values  q,k,v,out x (seq, batch);
+ * bwd 16 values: the same 8, then dout, dq, dk, dv x (seq, batch). */
+int ezl_attn_fwd(const void* q, const void* k, const void* v, void* out, void* lse, const void* cu_seqlens, int64_t ndocs,
+                 int64_t total_tokens, int64_t s_len, int64_t nq, int64_t nk, int64_t d, float scale, const int64_t* strides,
+                 void* stream);
+int ezl_attn_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout, const void* lse, void* delta,
+                 void* dq, void* dk, void* dv, const void* cu_seqlens, int64_t ndocs, int64_t total_tokens, int64_t s_len,
+                 int64_t nq, int64_t nk, int64_t d, float scale, const int64_t* strides, void* stream);
+
+/* ---- loss: base_modules/functions/cross_entropy.py:24-112 and llama/losses.py:20-56 ----
+ * logits [rows, vocab] bf16 (dtype 0) or fp32 (dtype 1); labels int64 [rows]; a label outside
+ * [0, vocab - cut_size) is masked exactly as the reference does (pred = 0, no one-hot).
+ * prepare: weights[i] = loss_mask[i] * (labels[i] != ignore_index), count[0] = sum(weights);
+ *          mask_dtype 0 none(=1), 1 fp32, 2 bool/uint8, 3 int64, 4 bf16.
+ * fwd/bwd: the reference's per-token autograd function split in two (loss + logsumexp; grad).
+ * fused:   loss rows and grad = (softmax - onehot) * weights / count in ONE visit (grad may alias logits).
+ * reduce:  loss_out[0] = sum(loss_rows * weights) / count[0]. */
+int ezl_ce_prepare(const void* labels, const void* loss_mask, int mask_dtype, int64_t ignore_index, void* weights, void* count,
+                   int64_t n, void* stream);
+int ezl_ce_fwd(const void* logits, const void* labels, void* loss, void* lse, int64_t rows, int64_t vocab, int64_t cut_size,
+               int dtype, void* stream);
+int ezl_ce_bwd(const void* logits, const void* labels, const void* lse, const void* grad_out, void* grad, int64_t rows,
+               int64_t vocab, int64_t cut_size, int dtype, void* stream);
+int ezl_ce_fused(const void* logits, const void* labels, const void* weights, const void* count, void* loss_rows, void* grad,
+                 int64_t rows, int64_t vocab, int64_t cut_size, int dtype, void* stream);
+int ezl_ce_reduce(const void* loss_rows, const void* weights, const void* count, void* loss_out, int64_t n, void* stream);
+/* x *= scalar[0] unless scalar[0] == 1 (applies the upstream gradient of the fused loss) */
+int ezl_scale_by_scalar(void* x, const void* scalar_f32, int64_t n, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
