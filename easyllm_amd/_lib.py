@@ -25,6 +25,8 @@ SIGNATURES = {
     "ezl_add": [_vp, _vp, _vp, _i64, _vp],
     "ezl_cast_bf16_to_f32": [_vp, _vp, _i64, _vp],
     "ezl_cast_f32_to_bf16": [_vp, _vp, _i64, _vp],
+    "ezl_bias_add": [_vp, _vp, _vp, _i64, _i64, _vp],
+    "ezl_bias_grad": [_vp, _vp, _vp, _i32, _vp, _i64, _i64, _i64, _vp],
     "ezl_gemm_bf16": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
     "ezl_attn_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64p, _vp],
     "ezl_attn_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32,
@@ -40,6 +42,7 @@ _SPECIAL = {
     "ezl_version": ([], ctypes.c_int),
     "ezl_last_error": ([], ctypes.c_char_p),
     "ezl_rmsnorm_bwd_workspace_bytes": ([_i64, _i64], _i64),
+    "ezl_bias_grad_workspace_bytes": ([_i64, _i64], _i64),
 }
 
 _lib = None
@@ -81,3 +84,7 @@ def call(name, *args):
 
 def rmsnorm_bwd_workspace_bytes(rows, h):
     return load().ezl_rmsnorm_bwd_workspace_bytes(rows, h)
+
+
+def bias_grad_workspace_bytes(rows, n):
+    return load().ezl_bias_grad_workspace_bytes(rows, n)

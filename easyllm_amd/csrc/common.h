@@ -73,4 +73,24 @@ __device__ __forceinline__ float wave_max(float v) {
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
     return v;
 }
+
+// out[col] (+)= sum_r partial[r][col];  64 columns per block, 4 row groups folded through LDS.
+template <int UNUSED>
+__global__ __launch_bounds__(256) void ezl_colsum_kernel(const float* __restrict__ partial, int nrows, int ncols,
+                                                     bf16_t* __restrict__ out_bf16, float* __restrict__ out_f32,
+                                                     int accumulate) {
+    __shared__ float s[4][64];
+    const int c = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int col = blockIdx.x * 64 + c;
+    float acc = 0.f;
+    if (col < ncols)
+        for (int r = g; r < nrows; r += 4) acc += partial[(size_t)r * ncols + col];
+    s[g][c] = acc;
+    __syncthreads();
+    if (g == 0 && col < ncols) {
+        const float v = s[0][c] + s[1][c] + s[2][c] + s[3][c];
+        if (out_f32) out_f32[col] = accumulate ? out_f32[col] + v : v;
+        else out_bf16[col] = (bf16_t)v;
+    }
+}
 #endif

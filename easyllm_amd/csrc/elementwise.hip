@@ -191,6 +191,38 @@ __global__ __launch_bounds__(kBlock) void f32_to_bf16_kernel(const float* __rest
     }
 }
 
+// out[r, :] = x[r, :] + bias   (column_parallel_linear.py:43-44)
+__global__ __launch_bounds__(kBlock) void bias_add_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ bias,
+                                                          bf16_t* __restrict__ out, int64_t rows, int n) {
+    const int n8 = n >> 3;
+    const int64_t items = rows * n8;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < items; i += (int64_t)gridDim.x * kBlock) {
+        const int c = (int)(i % n8);
+        float a[8], b[8];
+        unpack8(ld_bf16x8(x + i * 8), a);
+        unpack8(ld_bf16x8(bias + c * 8), b);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) a[k] += b[k];
+        st_bf16x8(out + i * 8, pack8(a));
+    }
+}
+
+// partial[blockIdx.y][col] = sum over rows r = blockIdx.y, blockIdx.y + gridDim.y, ... of dy[r][col]   (:100)
+__global__ __launch_bounds__(kBlock) void bias_grad_partial_kernel(const bf16_t* __restrict__ dy, float* __restrict__ partial,
+                                                                   int64_t rows, int n) {
+    const int col = (blockIdx.x * kBlock + threadIdx.x) * 8;
+    if (col >= n) return;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+        float v[8];
+        unpack8(ld_bf16x8(dy + r * n + col), v);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc[k] += v[k];
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) partial[(int64_t)blockIdx.y * n + col + k] = acc[k];
+}
+
 }  // namespace
 
 extern "C" int ezl_swiglu_fwd(const void* gate, const void* up, void* out, int64_t n, void* stream) {
@@ -316,5 +348,37 @@ extern "C" int ezl_cast_f32_to_bf16(const void* in, void* out, int64_t n, void* 
     hipLaunchKernelGGL(f32_to_bf16_kernel, dim3(grid_for(n / 8, kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
                        (const float*)in, (bf16_t*)out, n / 8);
     EZL_LAUNCH_CHECK("ezl_cast_f32_to_bf16");
+    return EZL_OK;
+}
+
+extern "C" int ezl_bias_add(const void* x, const void* bias, void* out, int64_t rows, int64_t n, void* stream) {
+    EZL_REQUIRE(rows >= 0 && n > 0 && n % 8 == 0 && n < (1LL << 31), EZL_EUNSUPPORTED, "ezl_bias_add: n must be a multiple of 8");
+    EZL_REQUIRE((rows == 0 || (x && bias && out)) && ezl_aligned16(x) && ezl_aligned16(bias) && ezl_aligned16(out), EZL_EINVAL,
+                "ezl_bias_add: null or misaligned pointer");
+    if (rows == 0) return EZL_OK;
+    hipLaunchKernelGGL(bias_add_kernel, dim3(grid_for(rows * (n / 8), kBlock)), dim3(kBlock), 0, (hipStream_t)stream,
+                       (const bf16_t*)x, (const bf16_t*)bias, (bf16_t*)out, rows, (int)n);
+    EZL_LAUNCH_CHECK("ezl_bias_add");
+    return EZL_OK;
+}
+
+extern "C" int64_t ezl_bias_grad_workspace_bytes(int64_t rows, int64_t n) {
+    (void)rows;
+    return (int64_t)64 * n * (int64_t)sizeof(float);
+}
+
+extern "C" int ezl_bias_grad(const void* dy, void* db_bf16, void* db_f32, int accumulate, void* workspace,
+                             int64_t workspace_bytes, int64_t rows, int64_t n, void* stream) {
+    EZL_REQUIRE(rows >= 0 && n > 0 && n % 8 == 0 && n < (1LL << 31), EZL_EUNSUPPORTED, "ezl_bias_grad: n must be a multiple of 8");
+    EZL_REQUIRE(dy && workspace && ezl_aligned16(dy) && ((db_bf16 != nullptr) != (db_f32 != nullptr)), EZL_EINVAL,
+                "ezl_bias_grad: bad pointer arguments");
+    EZL_REQUIRE(workspace_bytes >= ezl_bias_grad_workspace_bytes(rows, n), EZL_EINVAL, "ezl_bias_grad: workspace too small");
+    const dim3 grid((unsigned)((n / 8 + kBlock - 1) / kBlock), 64);
+    hipLaunchKernelGGL(bias_grad_partial_kernel, grid, dim3(kBlock), 0, (hipStream_t)stream, (const bf16_t*)dy, (float*)workspace,
+                       rows, (int)n);
+    EZL_LAUNCH_CHECK("ezl_bias_grad");
+    hipLaunchKernelGGL(ezl_colsum_kernel<0>, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, (hipStream_t)stream,
+                       (const float*)workspace, 64, (int)n, (bf16_t*)db_bf16, (float*)db_f32, accumulate);
+    EZL_LAUNCH_CHECK("ezl_bias_grad(colsum)");
     return EZL_OK;
 }

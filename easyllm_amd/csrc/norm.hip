@@ -170,25 +170,6 @@ __global__ __launch_bounds__(1024) void rmsnorm_bwd_kernel(const bf16_t* __restr
     for (int j = threadIdx.x; j < h; j += 1024) dw_partial[(size_t)blockIdx.x * h + j] = fold[j];
 }
 
-// out[col] (+)= sum_r partial[r][col];  64 columns per block, 4 row groups folded through LDS.
-__global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ partial, int nrows, int ncols,
-                                                     bf16_t* __restrict__ out_bf16, float* __restrict__ out_f32,
-                                                     int accumulate) {
-    __shared__ float s[4][64];
-    const int c = threadIdx.x & 63, g = threadIdx.x >> 6;
-    const int col = blockIdx.x * 64 + c;
-    float acc = 0.f;
-    if (col < ncols)
-        for (int r = g; r < nrows; r += 4) acc += partial[(size_t)r * ncols + col];
-    s[g][c] = acc;
-    __syncthreads();
-    if (g == 0 && col < ncols) {
-        const float v = s[0][c] + s[1][c] + s[2][c] + s[3][c];
-        if (out_f32) out_f32[col] = accumulate ? out_f32[col] + v : v;
-        else out_bf16[col] = (bf16_t)v;
-    }
-}
-
 int tpr_for(int h) {
     int t = (h / 8 + 63) / 64 * 64;
     return t < 64 ? 64 : (t > 256 ? 256 : t);
@@ -266,7 +247,7 @@ extern "C" int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight
     }
 #undef LAUNCH
     EZL_LAUNCH_CHECK("ezl_rmsnorm_bwd");
-    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((h + 63) / 64)), dim3(256), 0, st, (const float*)workspace,
+    hipLaunchKernelGGL(ezl_colsum_kernel<0>, dim3((unsigned)((h + 63) / 64)), dim3(256), 0, st, (const float*)workspace,
                        (int)grid, (int)h, (bf16_t*)dw_bf16, (float*)dw_f32, accumulate);
     EZL_LAUNCH_CHECK("ezl_rmsnorm_bwd(colsum)");
     return EZL_OK;

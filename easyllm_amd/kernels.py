@@ -208,6 +208,27 @@ def linear_wgrad(dy2d, x2d, out=None, accumulate=False):
     return gemm(dy2d, x2d, dy2d.shape[1], x2d.shape[1], dy2d.shape[0], lda, ldb, False, False, out=out, accumulate=accumulate)
 
 
+def bias_add(x, bias):
+    _bf16c(x, "x"); _bf16c(bias, "bias")
+    n = x.shape[-1]
+    _need(bias.numel() == n, "bias size mismatch")
+    out = torch.empty_like(x)
+    _lib.call("ezl_bias_add", _p(x), _p(bias), _p(out), x.numel() // n, n, _stream())
+    return out
+
+
+def bias_grad(dy, main_grad=None, accumulate=False):
+    """Column sum of dy [rows, n]: bf16 [n], or written into an fp32 main_grad (then returns None)."""
+    _bf16c(dy, "dy")
+    n = dy.shape[-1]
+    rows = dy.numel() // n
+    ws_bytes = _lib.bias_grad_workspace_bytes(rows, n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dy.device)
+    db = None if main_grad is not None else torch.empty(n, dtype=BF16, device=dy.device)
+    _lib.call("ezl_bias_grad", _p(dy), _p(db), _p(main_grad), 1 if accumulate else 0, _p(ws), ws_bytes, rows, n, _stream())
+    return db
+
+
 # ------------------------------------------------------------------------------------- attention
 def _tok_strides(t, b):
     """(seq_stride, batch_stride) of a [s, b, heads, d] tensor whose heads*d block is contiguous."""

@@ -78,6 +78,13 @@ int ezl_cast_f32_to_bf16(const void* in, void* out, int64_t n, void* stream);
 int ezl_gemm_bf16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                   int a_kc, int b_kc, int out_dtype, int accumulate, void* stream);
 
+/* bias of a linear layer: column_parallel_linear.py:43-44 (out = x + bias) and :100 (db = sum_rows dy);
+ * db goes to exactly one of db_bf16 [n] or db_f32 [n] (added to when accumulate != 0). */
+int ezl_bias_add(const void* x, const void* bias, void* out, int64_t rows, int64_t n, void* stream);
+int64_t ezl_bias_grad_workspace_bytes(int64_t rows, int64_t n);
+int ezl_bias_grad(const void* dy, void* db_bf16, void* db_f32, int accumulate, void* workspace, int64_t workspace_bytes,
+                  int64_t rows, int64_t n, void* stream);
+
 /* ---- attention: FlashAttention.forward, llama/transformer.py:83-143 (flash_attn_varlen_* seams
  *      :106-115) ----
  * q [T, nq, d], k/v [T, nk, d] bf16, d in {64, 128}; token n lives at
