@@ -1,0 +1,126 @@
+#!/usr/bin/env python3
+"""Benchmark of the llama decoder-layer training step (fwd + loss + bwd) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--no-cpu-baseline]
+
+Prints ONE JSON line.  A step = one forward + cross-entropy loss + backward of the workload's layer
+stack on one micro-batch of synthetic, HBM-resident inputs (random-init weights, seeded token ids);
+weight gradients land in fp32 main-grad buffers.  `value` = tokens / second of whole steps.
+`roofline` describes the dominant kernel (the bf16 MFMA GEMM): its algorithmic FLOPs divided by its
+launch durations, both taken inside the timed region with events on the launch stream.
+`cpu_baseline` = the fp32 CPU oracle (a port of the reference math) timed on this host's cores on a
+bounded sample (one decoder layer + LM head + loss of the same workload), extrapolated linearly.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "fwd+bwd tokens/sec + MFMA util %, 7B-shape llama layer bf16 seq4096, 1 GPU"
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak
+
+
+def cpu_baseline(w, budget_note=True):
+    """fp32 oracle on the host: one decoder layer + final norm + LM head + loss, fwd+bwd, then
+    t_step ~= L * t_layer + t_head.  Returns the dict that goes into the JSON line."""
+    import torch
+    from oracle import llama_oracle as O
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    b, s, h, V, L = w["batch"], w["seq"], w["hidden_size"], w["vocab_size"], w["num_layers"]
+    cfg = dict(num_layers=1, hidden_size=h, num_attention_heads=w["num_attention_heads"],
+               num_kv_attention_heads=w["num_kv_attention_heads"], head_dim=h // w["num_attention_heads"],
+               intermediate_size=w["intermediate_size"], vocab_size=V)
+    Wt = {k: v.requires_grad_(True) for k, v in O.init_weights(cfg, seed=1).items()}
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(s, b, h, generator=g).requires_grad_(True)
+    labels = torch.randint(0, V, (b, s), generator=g)
+    t0 = time.perf_counter()
+    y = O.decoder_layer(x, Wt, "3.", cfg)
+    y.backward(torch.ones_like(y))
+    t_layer = time.perf_counter() - t0
+    xh = torch.randn(b, s, h, generator=g).requires_grad_(True)
+    t0 = time.perf_counter()
+    logits = O.linear(O.rmsnorm(xh, Wt["5.weight"]), Wt["6.word_embeddings.weight"])
+    loss = O.cross_entropy_loss(logits, labels, torch.ones(b, s))
+    loss.backward()
+    t_head = time.perf_counter() - t0
+    t_step = L * t_layer + t_head
+    return {"value": round(b * s / t_step, 2), "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": "fp32 CPU oracle, 1 of %d decoder layers (%.1f s) + final norm/LM head/loss (%.1f s) fwd+bwd at the "
+                      "full shape; step time extrapolated as L*t_layer + t_head" % (L, t_layer, t_head)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="C2")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU's share only (TP=1, one MI355X); --gpus %d is not supported. "
+              "Run with --gpus 1." % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from easyllm_amd import kernels, runner, workloads as W
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = W.WORKLOADS[args.workload]
+    torch.manual_seed(w["seed"])
+    model = runner.build_model({"type": "llama_custom", "kwargs": W.model_kwargs(w)})
+    runner.attach_main_grads(model)
+    inputs, labels, doc_lens = W.make_inputs(w, device=dev)
+    tokens_per_step = w["batch"] * w["seq"]
+    flops = W.step_flops(w, doc_lens)
+
+    def step():
+        runner.zero_main_grads(model)
+        return runner.forward_step(model, inputs, labels)
+
+    for _ in range(args.warmup):
+        loss = step()
+    torch.cuda.synchronize()
+    kernels.GEMM_TIMING = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    timing, kernels.GEMM_TIMING = kernels.GEMM_TIMING, None
+    loss_value = float(loss.item())
+
+    ms_per_step = elapsed / args.steps * 1e3
+    tok_s = tokens_per_step * args.steps / elapsed
+    tflops = flops * args.steps / elapsed / 1e12
+    gemm_flops = sum(f for f, _, _ in timing)
+    gemm_ms = sum(s.elapsed_time(e) for _, s, e in timing)
+    gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12 if gemm_ms > 0 else 0.0
+    out = {
+        "metric": METRIC, "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "%s: %s" % (args.workload, w["desc"]), "tokens_per_step": tokens_per_step,
+                   "fp32_main_grads": True, "recomputed_layers": model.recompute_count},
+        "tflops": round(tflops, 1), "mfma_frac_end_to_end": round(tflops / PEAK_BF16_TFLOPS, 4), "loss": round(loss_value, 5),
+        "roofline": {"kernel": "gemm_kernel (bf16 MFMA GEMM, %d launches/step)" % (len(timing) // max(args.steps, 1)),
+                     "bound": "mfma", "achieved": round(gemm_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(gemm_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "share_of_step_time": round(gemm_ms / (elapsed * 1e3), 4)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -177,7 +177,24 @@ def _rows_ld(t, name):
     return t.stride(0)
 
 
+# Optional per-launch timing of the GEMM kernel (used by bench.py for the roofline figure): when a list
+# is installed here every launch is bracketed by two events on the launch stream and
+# (flops, start, end) is appended to it.
+GEMM_TIMING = None
+
+
 def gemm(A, B, M, N, K, lda, ldb, a_kc, b_kc, out=None, out_dtype=BF16, accumulate=False):
+    if GEMM_TIMING is not None:
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        out = _gemm(A, B, M, N, K, lda, ldb, a_kc, b_kc, out, out_dtype, accumulate)
+        end.record()
+        GEMM_TIMING.append((2.0 * M * N * K, start, end))
+        return out
+    return _gemm(A, B, M, N, K, lda, ldb, a_kc, b_kc, out, out_dtype, accumulate)
+
+
+def _gemm(A, B, M, N, K, lda, ldb, a_kc, b_kc, out, out_dtype, accumulate):
     if out is None:
         out = torch.empty(M, N, dtype=out_dtype, device=A.device)
     _need(out.is_cuda and out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (M, N), "bad GEMM output")
