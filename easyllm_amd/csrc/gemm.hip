@@ -7,20 +7,26 @@
 //   dgrad     dX[T,in]  = dY[T,out] * W[out,in]      A k-contiguous, B n-contiguous
 //   wgrad     dW[out,in]= dY[T,out]^T * X[T,in]      A m-contiguous, B n-contiguous   (fp32 or bf16 out)
 //
-// Tiling: 256x256 block tile, K step 64, 4 waves (2x2), each wave owns 128x128 = 4x4 MFMA
-// 32x32x16 tiles (256 fp32 accumulators per lane).  Both operand tiles are staged in LDS, double
-// buffered (2 x 2 x 36 KiB of the 160 KiB), filled through registers with 128-bit global loads that
-// are issued one full K step ahead of their use.  A k-contiguous operand is stored [row][64 + 8 pad]
-// and read with ds_read_b128; an operand whose reduction dimension is the strided one is stored as
-// it lies in memory, [k][256 + 32 pad], and read with ds_read_b64_tr_b16 (the LDS transpose read),
-// so no operand is ever transposed in HBM.  Blocks are renumbered so that each XCD (own L2) works
-// on a contiguous band of tiles, grouped 8 tiles tall.
+// Tiling: 256x256 block tile, K step 64, 8 waves (2x4), each wave owns 128x64 = 4x2 MFMA 32x32x16
+// tiles.  Operand tiles are double buffered in LDS (2 stages x 2 operands x 32 KiB).  An operand whose
+// reduction dimension is the strided one is kept as it lies in memory ([k][256]) and read with
+// ds_read_b64_tr_b16 (the LDS transpose read), so nothing is ever transposed in HBM.
+//
+// Main kernel (K % 64 == 0): tiles go HBM -> LDS directly (global_load_lds_dwordx4, no staging
+// registers, no ds_write); bank conflicts are avoided by an XOR swizzle applied on the global-address
+// side.  The K loop is rotated: the barrier that publishes the next stage sits between the fragment
+// reads and the MFMAs of the last 16-wide sub-step, so the loads of tile kt+2 and the first fragment
+// reads of tile kt+1 are issued under those MFMAs; scheduler group barriers interleave one LDS read
+// per two MFMAs.  A second kernel with register staging and padded tiles covers K tails (K % 64 != 0).
+// Blocks are renumbered so that each XCD (own L2) works on a contiguous band of tiles, 8 tiles tall.
 #include "common.h"
 
 namespace {
 
+// =================================================================================================
+// K-tail kernel: register-staged loads, padded tiles
+// =================================================================================================
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int NT = 256;
 constexpr int LDK = BK + 8;     // row stride (elements) of a k-contiguous tile  [256][72]
 constexpr int LDN = 256 + 32;   // row stride (elements) of a k-major tile       [64][288]
 constexpr int TILE = 256 * LDK; // == 64 * LDN elements per operand per stage
@@ -28,46 +34,53 @@ static_assert(TILE == 64 * LDN, "both tile layouts must have the same footprint"
 
 typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
 
-// ---- global -> register staging of one operand tile (8 x 128-bit per thread) -------------------
-template <bool KC>
+// ---- global -> register staging of one operand tile (2048 x 128-bit chunks over NT threads) ----
+template <bool KC, int NT, bool KTAIL>
 struct Stager {
-    uint32_t off[8];  // element offsets of this thread's 8 chunks at k = 0
-    int krow;         // (non-KC) k row of chunk 0 / (KC) k column of all chunks
+    static constexpr int NCH = 2048 / NT;   // chunks per thread
+    static constexpr int RSTEP = NT / 8;    // KC: tile rows between two chunks of a thread
+    static constexpr int KSTEP = NT / 32;   // non-KC: k rows between two chunks of a thread
+    uint32_t off[NCH];  // element offsets of this thread's chunks at k = 0
+    int kpos;           // (KC) k column of all chunks / (non-KC) k row of chunk 0
     // dim = extent of the non-reduction dimension, first = first row/col of the block tile
     __device__ __forceinline__ void init(int tid, int first, int dim, int64_t ld) {
         if (KC) {
-            krow = (tid & 7) * 8;
+            kpos = (tid & 7) * 8;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                int r = first + (tid >> 3) + 32 * i;
-                r = r < dim ? r : dim - 1;
-                off[i] = (uint32_t)((int64_t)r * ld + krow);
+            for (int i = 0; i < NCH; ++i) {
+                int r = first + (tid >> 3) + RSTEP * i;
+                r = r < dim ? r : dim - 1;  // rows past the edge re-read the last row; their results are never stored
+                off[i] = (uint32_t)((int64_t)r * ld + kpos);
             }
         } else {
-            krow = tid >> 5;
+            kpos = tid >> 5;
             int c = first + (tid & 31) * 8;
             c = c + 8 <= dim ? c : dim - 8;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) off[i] = (uint32_t)((int64_t)(krow + 8 * i) * ld + c);
+            for (int i = 0; i < NCH; ++i) off[i] = (uint32_t)((int64_t)(kpos + KSTEP * i) * ld + c);
         }
     }
     // k0 = first k of the tile; kadv = element offset of that k (k0 for KC, k0 * ld otherwise)
     __device__ __forceinline__ void load(const bf16_t* __restrict__ base, int k0, int64_t kadv, int K, bf16x8* r) const {
         const bf16_t* p = base + kadv;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const bool ok = KC ? (k0 + krow < K) : (k0 + krow + 8 * i < K);
-            bf16x8 z;
+        for (int i = 0; i < NCH; ++i) {
+            if (KTAIL) {
+                const bool ok = KC ? (k0 + kpos < K) : (k0 + kpos + KSTEP * i < K);
+                bf16x8 z;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) z[j] = (bf16_t)0.0f;
-            r[i] = ok ? *reinterpret_cast<const bf16x8*>(p + off[i]) : z;
+                for (int j = 0; j < 8; ++j) z[j] = (bf16_t)0.0f;
+                r[i] = ok ? *reinterpret_cast<const bf16x8*>(p + off[i]) : z;
+            } else {
+                r[i] = *reinterpret_cast<const bf16x8*>(p + off[i]);
+            }
         }
     }
     __device__ __forceinline__ void store(bf16_t* __restrict__ s, int tid, const bf16x8* r) const {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            if (KC) *reinterpret_cast<bf16x8*>(s + ((tid >> 3) + 32 * i) * LDK + (tid & 7) * 8) = r[i];
-            else *reinterpret_cast<bf16x8*>(s + ((tid >> 5) + 8 * i) * LDN + (tid & 31) * 8) = r[i];
+        for (int i = 0; i < NCH; ++i) {
+            if (KC) *reinterpret_cast<bf16x8*>(s + ((tid >> 3) + RSTEP * i) * LDK + (tid & 7) * 8) = r[i];
+            else *reinterpret_cast<bf16x8*>(s + ((tid >> 5) + KSTEP * i) * LDN + (tid & 31) * 8) = r[i];
         }
     }
 };
@@ -99,13 +112,17 @@ template <> __device__ __forceinline__ void store_out<float>(float* p, float v, 
     *p = accumulate ? v + *p : v;
 }
 
-template <bool A_KC, bool B_KC, typename OutT>
-__global__ __launch_bounds__(NT) void gemm_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B, OutT* __restrict__ C,
-                                                  int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
-                                                  int tiles_m, int tiles_n) {
+// WAVES_M x WAVES_N waves tile the 256x256 block; a wave owns (256/WAVES_M) x (256/WAVES_N)
+template <bool A_KC, bool B_KC, typename OutT, bool KTAIL, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_staged_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
+                                                                      OutT* __restrict__ C, int M, int N, int K, int64_t lda,
+                                                                      int64_t ldb, int64_t ldc, int accumulate, int tiles_m,
+                                                                      int tiles_n) {
+    constexpr int NT = WAVES_M * WAVES_N * 64;
+    constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;  // MFMA tiles per wave
     __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TILE];  // A0 B0 A1 B1
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
     // XCD-aware renumbering: hardware deals consecutive block ids round-robin to the 8 XCDs
     const int nblocks = tiles_m * tiles_n;
@@ -123,17 +140,18 @@ __global__ __launch_bounds__(NT) void gemm_kernel(const bf16_t* __restrict__ A, 
     const int tn = (pid % group_size) / gm;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    Stager<A_KC> sa;
-    Stager<B_KC> sb;
+    Stager<A_KC, NT, KTAIL> sa;
+    Stager<B_KC, NT, KTAIL> sb;
     sa.init(tid, m0, M, lda);
     sb.init(tid, n0, N, ldb);
-    bf16x8 ra[8], rb[8];
+    constexpr int NCH = 2048 / NT;
+    bf16x8 ra[NCH], rb[NCH];
 
-    f32x16 acc[4][4];
+    f32x16 acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
@@ -153,8 +171,8 @@ __global__ __launch_bounds__(NT) void gemm_kernel(const bf16_t* __restrict__ A, 
 
     for (int kt = 0; kt < nk; ++kt) {
         const int cur = kt & 1;
-        bf16_t* sA = smem + cur * 2 * TILE;
-        bf16_t* sB = sA + TILE;
+        const bf16_t* sA = smem + cur * 2 * TILE;
+        const bf16_t* sB = sA + TILE;
         if (kt + 1 < nk) {  // tile kt+1 sits in registers: park it in the other stage
             sa.store(smem + (cur ^ 1) * 2 * TILE, tid, ra);
             sb.store(smem + (cur ^ 1) * 2 * TILE + TILE, tid, rb);
@@ -165,15 +183,15 @@ __global__ __launch_bounds__(NT) void gemm_kernel(const bf16_t* __restrict__ A, 
         }
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 fa[4], fb[4];
+            bf16x8 fa[TM], fb[TN];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fa[i] = frag<A_KC>(sA, wm * 128 + i * 32, ks, lane);
+            for (int i = 0; i < TM; ++i) fa[i] = frag<A_KC>(sA, wm * (TM * 32) + i * 32, ks, lane);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) fb[j] = frag<B_KC>(sB, wn * 128 + j * 32, ks, lane);
+            for (int j = 0; j < TN; ++j) fb[j] = frag<B_KC>(sB, wn * (TN * 32) + j * 32, ks, lane);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
         }
         __syncthreads();
@@ -181,20 +199,226 @@ __global__ __launch_bounds__(NT) void gemm_kernel(const bf16_t* __restrict__ A, 
 
     // epilogue: lane holds column (lane & 31); register r is row 8*(r/4) + 4*(lane>>5) + r%4
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int col = n0 + wn * 128 + j * 32 + (lane & 31);
+        for (int j = 0; j < TN; ++j) {
+            const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const int row = m0 + wm * (TM * 32) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (row < M && col < N) store_out<OutT>(C + (int64_t)row * ldc + col, acc[i][j][r], accumulate != 0);
             }
         }
     }
 }
 
+
+// =================================================================================================
+// main kernel: direct-to-LDS loads, XOR-swizzled tiles
+// =================================================================================================
+constexpr int DTILE = 256 * 64;  // elements per operand per stage of the swizzled layout (32 KiB)
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(1))) const void gvoid;
+
+#define SG_MFMA 0x008
+#define SG_VMEM_R 0x020
+#define SG_DS_R 0x100
+
+// One operand tile = 32 wave-instructions of 1 KiB each (global_load_lds_dwordx4: lane l lands at base + 16 l).
+//   k-contiguous tile [256 rows][64 k]:  instruction q covers rows 8q..8q+7; chunk c of row r sits in slot c ^ ((r>>1)&7)
+//   k-major tile      [64 k][256 cols]:  instruction q covers k rows 2q, 2q+1; chunk c of k row sits in slot c ^ ((k&3)<<2)
+template <bool KC, int NW>
+struct Loader {
+    static constexpr int NI = 32 / NW;
+    uint32_t off[NI];
+    __device__ __forceinline__ void init(int lane, int wave, int first, int dim, int64_t ld) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int q = wave + NW * i;
+            if (KC) {
+                const int row = 8 * q + (lane >> 3);
+                const int c = (lane & 7) ^ ((row >> 1) & 7);
+                int gr = first + row;
+                gr = gr < dim ? gr : dim - 1;
+                off[i] = (uint32_t)((int64_t)gr * ld + c * 8);
+            } else {
+                const int krow = 2 * q + (lane >> 5);
+                const int c = (lane & 31) ^ ((krow & 3) << 2);
+                int col = first + c * 8;
+                col = col + 8 <= dim ? col : dim - 8;
+                off[i] = (uint32_t)((int64_t)krow * ld + col);
+            }
+        }
+    }
+    __device__ __forceinline__ void issue(const bf16_t* __restrict__ gbase, bf16_t* stage, int wave) const {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int q = wave + NW * i;
+            __builtin_amdgcn_global_load_lds((gvoid*)(gbase + off[i]), (lds_void*)(stage + q * 512), 16, 0, 0);
+        }
+    }
+};
+
+template <bool KC>
+__device__ __forceinline__ bf16x8 sfrag(const bf16_t* __restrict__ s, int row0, int ks, int lane) {
+    if (KC) {
+        const int row = row0 + (lane & 31);
+        const int c = (ks * 2 + (lane >> 5)) ^ ((row >> 1) & 7);
+        return *reinterpret_cast<const bf16x8*>(s + row * 64 + c * 8);
+    } else {
+        const int q = lane >> 4;
+        const int krow = ks * 16 + (q >> 1) * 8 + ((lane & 15) >> 2);
+        const int col = row0 + (q & 1) * 16 + ((lane & 3) << 2);
+        const int c = (col >> 3) ^ ((krow & 3) << 2);
+        const bf16_t* p = s + krow * 256 + c * 8 + (col & 7);
+        const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p));
+        const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p + 4 * 256));
+        bf16x8 v;
+        v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
+        v[4] = hi[0]; v[5] = hi[1]; v[6] = hi[2]; v[7] = hi[3];
+        return v;
+    }
+}
+
+template <bool A_KC, bool B_KC, typename OutT, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_d2l_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
+                                                                          OutT* __restrict__ C, int M, int N, int K, int64_t lda,
+                                                                          int64_t ldb, int64_t ldc, int accumulate, int tiles_m,
+                                                                          int tiles_n) {
+    constexpr int NW = WAVES_M * WAVES_N;
+    constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
+    constexpr int NKS = BK / 16;
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[4 * DTILE];  // A0 B0 A1 B1
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+    const int nblocks = tiles_m * tiles_n;
+    int pid = blockIdx.x;
+    {
+        const int per = nblocks >> 3, rem = nblocks & 7, xcd = pid & 7, idx = pid >> 3;
+        pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    }
+    constexpr int GROUP_M = 8;
+    const int group_size = GROUP_M * tiles_n;
+    const int group = pid / group_size;
+    const int first_m = group * GROUP_M;
+    const int gm = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
+    const int tm = first_m + (pid % group_size) % gm;
+    const int tn = (pid % group_size) / gm;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    Loader<A_KC, NW> la;
+    Loader<B_KC, NW> lb;
+    la.init(lane, wave, m0, M, lda);
+    lb.init(lane, wave, n0, N, ldb);
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int nk = K / BK;
+    const int64_t astep = A_KC ? BK : (int64_t)BK * lda;
+    const int64_t bstep = B_KC ? BK : (int64_t)BK * ldb;
+    const int arow = wm * (TM * 32), brow = wn * (TN * 32);
+
+    bf16x8 fa[2][TM], fb[2][TN];
+    auto read_frags = [&](const bf16_t* sA, int ks, int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[buf][i] = sfrag<A_KC>(sA, arow + i * 32, ks, lane);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[buf][j] = sfrag<B_KC>(sA + DTILE, brow + j * 32, ks, lane);
+    };
+    auto mfmas = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+    };
+    auto issue_tile = [&](int t, int stage) {
+        la.issue(A + (int64_t)t * astep, smem + stage * 2 * DTILE, wave);
+        lb.issue(B + (int64_t)t * bstep, smem + stage * 2 * DTILE + DTILE, wave);
+    };
+
+    issue_tile(0, 0);
+    if (nk > 1) issue_tile(1, 1);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+    read_frags(smem, 0, 0);
+
+    constexpr int RD = (A_KC ? TM : 2 * TM) + (B_KC ? TN : 2 * TN);  // LDS reads per sub-step
+#define EZL_STEP(HAS_NEXT, DO_LOAD)                                                                       \
+    {                                                                                                     \
+        const int cur = kt & 1;                                                                           \
+        const bf16_t* sA = smem + cur * 2 * DTILE;                                                         \
+        _Pragma("unroll") for (int ks = 0; ks < NKS - 1; ++ks) {                                          \
+            read_frags(sA, ks + 1, (ks + 1) & 1);                                                         \
+            mfmas(ks & 1);                                                                                \
+            _Pragma("unroll") for (int g = 0; g < TM * TN / 2; ++g) {                                     \
+                __builtin_amdgcn_sched_group_barrier(SG_MFMA, 2, 0);                                      \
+                __builtin_amdgcn_sched_group_barrier(SG_DS_R, RD > TM * TN / 2 ? 2 : 1, 0);               \
+            }                                                                                             \
+        }                                                                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                                \
+        __builtin_amdgcn_s_waitcnt(0x0F70);                                                               \
+        __syncthreads();                                                                                  \
+        __builtin_amdgcn_sched_barrier(0);                                                                \
+        if (DO_LOAD) issue_tile(kt + 2, cur);                                                             \
+        if (HAS_NEXT) read_frags(smem + (cur ^ 1) * 2 * DTILE, 0, 0);                                      \
+        mfmas((NKS - 1) & 1);                                                                             \
+        _Pragma("unroll") for (int g = 0; g < TM * TN / 2; ++g) {                                         \
+            __builtin_amdgcn_sched_group_barrier(SG_MFMA, 2, 0);                                          \
+            if (DO_LOAD) __builtin_amdgcn_sched_group_barrier(SG_VMEM_R, 2, 0);                           \
+            if (HAS_NEXT) __builtin_amdgcn_sched_group_barrier(SG_DS_R, RD > TM * TN / 2 ? 2 : 1, 0);     \
+        }                                                                                                 \
+        __builtin_amdgcn_sched_barrier(0);                                                                \
+    }
+
+    int kt = 0;
+    for (; kt + 2 < nk; ++kt) EZL_STEP(true, true)
+    if (kt + 1 < nk) {
+        EZL_STEP(true, false)
+        ++kt;
+    }
+    EZL_STEP(false, false)
+#undef EZL_STEP
+
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm * (TM * 32) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (row < M && col < N) store_out<OutT>(C + (int64_t)row * ldc + col, acc[i][j][r], accumulate != 0);
+            }
+        }
+    }
+}
+
+
+template <bool A_KC, bool B_KC, typename OutT>
+void launch(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
+            hipStream_t st) {
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const dim3 grid((unsigned)(tiles_m * tiles_n)), block(512);
+    if (K % BK == 0)
+        hipLaunchKernelGGL((gemm_d2l_kernel<A_KC, B_KC, OutT, 2, 4>), grid, block, 0, st, (const bf16_t*)A, (const bf16_t*)B,
+                           (OutT*)C, M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n);
+    else
+        hipLaunchKernelGGL((gemm_staged_kernel<A_KC, B_KC, OutT, true, 2, 4>), grid, block, 0, st, (const bf16_t*)A,
+                           (const bf16_t*)B, (OutT*)C, M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n);
+}
+
 }  // namespace
+
 
 // a_kc / b_kc: 1 if the operand's reduction index is its contiguous one
 //   A: a_kc ? A[m * lda + k] : A[k * lda + m]        B: b_kc ? B[n * ldb + k] : B[k * ldb + n]
@@ -215,25 +439,22 @@ extern "C" int ezl_gemm_bf16(const void* A, const void* B, void* C, int64_t M, i
     const int64_t a_rows = a_kc ? M : K, b_rows = b_kc ? N : K;
     EZL_REQUIRE(a_rows * lda < (1LL << 32) && b_rows * ldb < (1LL << 32) && M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31),
                 EZL_EUNSUPPORTED, "ezl_gemm_bf16: operand larger than 2^32 elements");
-    const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
-    EZL_REQUIRE((int64_t)tiles_m * tiles_n < (1LL << 31), EZL_EUNSUPPORTED, "ezl_gemm_bf16: too many tiles");
-    const dim3 grid((unsigned)(tiles_m * tiles_n)), block(NT);
+    const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    EZL_REQUIRE(tiles < (1LL << 31), EZL_EUNSUPPORTED, "ezl_gemm_bf16: too many tiles");
     hipStream_t st = (hipStream_t)stream;
-#define LAUNCH(AK, BKC, OT)                                                                                         \
-    hipLaunchKernelGGL((gemm_kernel<AK, BKC, OT>), grid, block, 0, st, (const bf16_t*)A, (const bf16_t*)B, (OT*)C, (int)M, \
-                       (int)N, (int)K, lda, ldb, ldc, accumulate, tiles_m, tiles_n)
+#define EZL_GEMM_CASE(AK, BKC, OT) launch<AK, BKC, OT>(A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, accumulate, st)
     if (out_dtype == 0) {
-        if (a_kc && b_kc) LAUNCH(true, true, bf16_t);
-        else if (a_kc && !b_kc) LAUNCH(true, false, bf16_t);
-        else if (!a_kc && !b_kc) LAUNCH(false, false, bf16_t);
-        else LAUNCH(false, true, bf16_t);
+        if (a_kc && b_kc) EZL_GEMM_CASE(true, true, bf16_t);
+        else if (a_kc && !b_kc) EZL_GEMM_CASE(true, false, bf16_t);
+        else if (!a_kc && !b_kc) EZL_GEMM_CASE(false, false, bf16_t);
+        else EZL_GEMM_CASE(false, true, bf16_t);
     } else {
-        if (a_kc && b_kc) LAUNCH(true, true, float);
-        else if (a_kc && !b_kc) LAUNCH(true, false, float);
-        else if (!a_kc && !b_kc) LAUNCH(false, false, float);
-        else LAUNCH(false, true, float);
+        if (a_kc && b_kc) EZL_GEMM_CASE(true, true, float);
+        else if (a_kc && !b_kc) EZL_GEMM_CASE(true, false, float);
+        else if (!a_kc && !b_kc) EZL_GEMM_CASE(false, false, float);
+        else EZL_GEMM_CASE(false, true, float);
     }
-#undef LAUNCH
+#undef EZL_GEMM_CASE
     EZL_LAUNCH_CHECK("ezl_gemm_bf16");
     return EZL_OK;
 }
