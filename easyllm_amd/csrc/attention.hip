@@ -46,7 +46,10 @@ __device__ __forceinline__ int64_t tok_off(int n, int s_len, int64_t ss, int64_t
     return (int64_t)b * sb + (int64_t)(n - b * s_len) * ss;
 }
 
-// block id -> (document, block inside the document); false if the id is beyond the last block
+// block id -> (document, block inside the document); false if the id is beyond the last block.
+// A document is cut at batch-row boundaries (the reference's collator never emits one that crosses a
+// row: it appends every row's length to that row's boundaries), so inside a document token i lives at
+// tok_off(doc_start) + i * seq_stride and no per-token division is needed.
 __device__ __forceinline__ bool find_block(const int* __restrict__ cu, int ndocs, int s_len, int T, int bid, int blk_rows,
                                            int& doc_start, int& doc_len, int& blk) {
     for (int d = 0; d < ndocs; ++d) {
@@ -54,16 +57,20 @@ __device__ __forceinline__ bool find_block(const int* __restrict__ cu, int ndocs
         int e = cu ? cu[d + 1] : (d + 1) * s_len;
         a = a < 0 ? 0 : a;
         e = e > T ? T : e;
-        const int len = e - a;
-        if (len <= 0) continue;
-        const int nb = (len + blk_rows - 1) / blk_rows;
-        if (bid < nb) {
-            doc_start = a;
-            doc_len = len;
-            blk = bid;
-            return true;
+        while (a < e) {
+            const int row_end = (a / s_len + 1) * s_len;
+            const int e1 = e < row_end ? e : row_end;
+            const int len = e1 - a;
+            const int nb = (len + blk_rows - 1) / blk_rows;
+            if (bid < nb) {
+                doc_start = a;
+                doc_len = len;
+                blk = bid;
+                return true;
+            }
+            bid -= nb;
+            a = e1;
         }
-        bid -= nb;
     }
     return false;
 }
@@ -76,19 +83,16 @@ struct Tile {
     static constexpr int NCH = ROWS * CH / kThreads;  // chunks per thread
     static constexpr int ELEMS = ROWS * LD;
 
-    // rows tok0 .. tok0+63 of head column hoff; rows at or beyond tok_end are zero
-    static __device__ __forceinline__ void load(const bf16_t* __restrict__ base, int64_t hoff, int tok0, int tok_end, int s_len,
-                                                int64_t ss, int64_t sb, int tid, bf16x8* r) {
+    // rows row0 .. row0+63 of a document whose token 0 (head column included) is at `base`; rows at or past
+    // doc_len re-read the document's last row: finite values that only ever meet masked (zero) probabilities
+    static __device__ __forceinline__ void load(const bf16_t* __restrict__ base, int64_t ss, int row0, int doc_len, int tid,
+                                                bf16x8* r) {
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             const int c = tid + kThreads * i;
-            const int row = c / CH, cc = c % CH;
-            const int n = tok0 + row;
-            bf16x8 z;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) z[j] = (bf16_t)0.0f;
-            r[i] = z;
-            if (n < tok_end) r[i] = *reinterpret_cast<const bf16x8*>(base + tok_off(n, s_len, ss, sb) + hoff + cc * 8);
+            int n = row0 + c / CH;
+            n = n < doc_len ? n : doc_len - 1;
+            r[i] = *reinterpret_cast<const bf16x8*>(base + (int64_t)n * ss + (c % CH) * 8);
         }
     }
     static __device__ __forceinline__ void store(bf16_t* __restrict__ s, int tid, const bf16x8* r) {
@@ -144,7 +148,7 @@ __device__ __forceinline__ void load_row_frags(const bf16_t* __restrict__ rowp, 
 // forward
 // =================================================================================================
 template <int D>
-__global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
     using TL = Tile<D>;
     __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS];  // K0 V0 K1 V1
     int doc_start, doc_len, qb;
@@ -162,14 +166,16 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
     const int kend = (q0 + 128 < doc_len ? q0 + 128 : doc_len);
     const int ntiles = (kend + 63) / 64;
     const int64_t kh = (int64_t)hk * D;
+    const bf16_t* kbase = p.k + tok_off(doc_start, p.s_len, p.k_ss, p.k_sb) + kh;
+    const bf16_t* vbase = p.v + tok_off(doc_start, p.s_len, p.v_ss, p.v_sb) + kh;
     bf16x8 rk[TL::NCH], rv[TL::NCH];
-    TL::load(p.k, kh, doc_start, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
-    TL::load(p.v, kh, doc_start, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+    TL::load(kbase, p.k_ss, 0, doc_len, tid, rk);
+    TL::load(vbase, p.v_ss, 0, doc_len, tid, rv);
     TL::store(smem, tid, rk);
     TL::store(smem + TL::ELEMS, tid, rv);
     if (ntiles > 1) {
-        TL::load(p.k, kh, doc_start + 64, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
-        TL::load(p.v, kh, doc_start + 64, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+        TL::load(kbase, p.k_ss, 64, doc_len, tid, rk);
+        TL::load(vbase, p.v_ss, 64, doc_len, tid, rv);
     }
     __syncthreads();
 
@@ -190,8 +196,8 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
             TL::store(smem + (cur ^ 1) * 2 * TL::ELEMS + TL::ELEMS, tid, rv);
         }
         if (t + 2 < ntiles) {
-            TL::load(p.k, kh, doc_start + (t + 2) * 64, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
-            TL::load(p.v, kh, doc_start + (t + 2) * 64, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+            TL::load(kbase, p.k_ss, (t + 2) * 64, doc_len, tid, rk);
+            TL::load(vbase, p.v_ss, (t + 2) * 64, doc_len, tid, rv);
         }
         const int key0 = t * 64;
         if (key0 <= qw0 + 31) {  // otherwise every key of the tile is after every query of this wave
@@ -205,35 +211,36 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
                     sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_kc(sK, kb * 32, kd, lane), qf[kd], sacc[kb], 0, 0, 0);
             }
             const bool need_mask = key0 + 63 > qw0;
-            float mloc = -INFINITY;
+            float mloc = -INFINITY;  // running maximum is kept on the raw (unscaled) scores
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    float s = sacc[kb][r] * sl2;
-                    if (need_mask && key0 + kb * 32 + acc_row(r, lane) > qi) s = -INFINITY;
-                    sacc[kb][r] = s;
-                    mloc = fmaxf(mloc, s);
+                    if (need_mask && key0 + kb * 32 + acc_row(r, lane) > qi) sacc[kb][r] = -INFINITY;
+                    mloc = fmaxf(mloc, sacc[kb][r]);
                 }
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
             const float mnew = fmaxf(m, mloc);
-            const float msafe = mnew == -INFINITY ? 0.f : mnew;
-            const float alpha = __builtin_amdgcn_exp2f(m - msafe);
+            const float moff = (mnew == -INFINITY ? 0.f : mnew) * sl2;
             float psum = 0.f;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const float pe = __builtin_amdgcn_exp2f(sacc[kb][r] - msafe);
+                    const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], sl2, -moff));
                     sacc[kb][r] = pe;
                     psum += pe;
                 }
-            lsum = lsum * alpha + psum;
+            if (__builtin_amdgcn_ballot_w64(mnew > m) != 0) {  // some query of this wave saw a new maximum
+                const float alpha = __builtin_amdgcn_exp2f(__builtin_fmaf(m, sl2, -moff));
+                lsum *= alpha;
+#pragma unroll
+                for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+            }
+            lsum += psum;
             m = mnew;
-#pragma unroll
-            for (int i = 0; i < D / 32; ++i)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -260,7 +267,7 @@ __global__ __launch_bounds__(kThreads) void attn_fwd_kernel(AttnParams p) {
                 for (int e = 0; e < 4; ++e) w[e] = (bf16_t)(oacc[db][r4 * 4 + e] * inv);
                 *reinterpret_cast<bf16x4*>(orow + db * 32 + 8 * r4 + 4 * (lane >> 5)) = w;
             }
-        if (lane < 32) p.lse[(int64_t)hq * p.T + doc_start + qi] = (m + __builtin_amdgcn_logf(ltot)) * kLn2;
+        if (lane < 32) p.lse[(int64_t)hq * p.T + doc_start + qi] = m * p.scale + __builtin_amdgcn_logf(ltot) * kLn2;
     }
 }
 
@@ -319,15 +326,17 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
     const int total = nqt * group;                // flattened (head in group, query tile) iterations
     const float sl2 = p.scale * kLog2e;
 
+    const bf16_t* qdoc = p.q + tok_off(doc_start, p.s_len, p.q_ss, p.q_sb);
+    const bf16_t* dodoc = p.dout + tok_off(doc_start, p.s_len, p.do_ss, p.do_sb);
     bf16x8 rq[TL::NCH], rdo[TL::NCH];
     float rstat = 0.f;  // threads 0..63: lse*log2e of query tid; 64..127: delta of query tid-64
     auto load_iter = [&](int it) {
         const int hq = hk * group + it / nqt;
-        const int tok0 = doc_start + (qt0 + it % nqt) * 64;
-        TL::load(p.q, (int64_t)hq * D, tok0, tok_end, p.s_len, p.q_ss, p.q_sb, tid, rq);
-        TL::load(p.dout, (int64_t)hq * D, tok0, tok_end, p.s_len, p.do_ss, p.do_sb, tid, rdo);
+        const int row0 = (qt0 + it % nqt) * 64;
+        TL::load(qdoc + (int64_t)hq * D, p.q_ss, row0, doc_len, tid, rq);
+        TL::load(dodoc + (int64_t)hq * D, p.do_ss, row0, doc_len, tid, rdo);
         if (tid < 128) {
-            const int n = tok0 + (tid & 63);
+            const int n = doc_start + row0 + (tid & 63);
             rstat = 0.f;
             if (n < tok_end) rstat = tid < 64 ? p.lse[(int64_t)hq * p.T + n] * kLog2e : p.delta[(int64_t)hq * p.T + n];
         }
@@ -416,7 +425,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
 // backward, dQ: a block owns 128 queries of one head and walks the keys at or before them
 // =================================================================================================
 template <int D>
-__global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(AttnParams p) {
+__global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) {
     using TL = Tile<D>;
     __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS];  // K0 V0 K1 V1
     int doc_start, doc_len, qb;
@@ -437,14 +446,16 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(AttnParams p) {
     const int kend = (q0 + 128 < doc_len ? q0 + 128 : doc_len);
     const int ntiles = (kend + 63) / 64;
     const int64_t kh = (int64_t)hk * D;
+    const bf16_t* kbase = p.k + tok_off(doc_start, p.s_len, p.k_ss, p.k_sb) + kh;
+    const bf16_t* vbase = p.v + tok_off(doc_start, p.s_len, p.v_ss, p.v_sb) + kh;
     bf16x8 rk[TL::NCH], rv[TL::NCH];
-    TL::load(p.k, kh, doc_start, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
-    TL::load(p.v, kh, doc_start, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+    TL::load(kbase, p.k_ss, 0, doc_len, tid, rk);
+    TL::load(vbase, p.v_ss, 0, doc_len, tid, rv);
     TL::store(smem, tid, rk);
     TL::store(smem + TL::ELEMS, tid, rv);
     if (ntiles > 1) {
-        TL::load(p.k, kh, doc_start + 64, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
-        TL::load(p.v, kh, doc_start + 64, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+        TL::load(kbase, p.k_ss, 64, doc_len, tid, rk);
+        TL::load(vbase, p.v_ss, 64, doc_len, tid, rv);
     }
     __syncthreads();
 
@@ -464,8 +475,8 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dq_kernel(AttnParams p) {
             TL::store(smem + (cur ^ 1) * 2 * TL::ELEMS + TL::ELEMS, tid, rv);
         }
         if (t + 2 < ntiles) {
-            TL::load(p.k, kh, doc_start + (t + 2) * 64, tok_end, p.s_len, p.k_ss, p.k_sb, tid, rk);
-            TL::load(p.v, kh, doc_start + (t + 2) * 64, tok_end, p.s_len, p.v_ss, p.v_sb, tid, rv);
+            TL::load(kbase, p.k_ss, (t + 2) * 64, doc_len, tid, rk);
+            TL::load(vbase, p.v_ss, (t + 2) * 64, doc_len, tid, rv);
         }
         const int key0 = t * 64;
         if (key0 <= qw0 + 31) {
@@ -539,7 +550,7 @@ extern "C" int ezl_attn_fwd(const void* q, const void* k, const void* v, void* o
     p.scale = scale;
     p.q_ss = strides[0]; p.q_sb = strides[1]; p.k_ss = strides[2]; p.k_sb = strides[3];
     p.v_ss = strides[4]; p.v_sb = strides[5]; p.o_ss = strides[6]; p.o_sb = strides[7];
-    const dim3 grid((unsigned)((total_tokens + 127) / 128 + ndocs), (unsigned)nq);
+    const dim3 grid((unsigned)((total_tokens + 127) / 128 + ndocs + total_tokens / s_len), (unsigned)nq);
     if (d == 128) hipLaunchKernelGGL(attn_fwd_kernel<128>, grid, dim3(kThreads), 0, (hipStream_t)stream, p);
     else hipLaunchKernelGGL(attn_fwd_kernel<64>, grid, dim3(kThreads), 0, (hipStream_t)stream, p);
     EZL_LAUNCH_CHECK("ezl_attn_fwd");
@@ -571,8 +582,8 @@ extern "C" int ezl_attn_bwd(const void* q, const void* k, const void* v, const v
     const int per_block = kThreads / (int)(d / 8);
     int64_t g = (items + per_block - 1) / per_block;
     if (g > 256 * 32) g = 256 * 32;
-    const dim3 gridq((unsigned)((total_tokens + 127) / 128 + ndocs), (unsigned)nq);
-    const dim3 gridk((unsigned)((total_tokens + 127) / 128 + ndocs), (unsigned)nk);
+    const dim3 gridq((unsigned)((total_tokens + 127) / 128 + ndocs + total_tokens / s_len), (unsigned)nq);
+    const dim3 gridk((unsigned)((total_tokens + 127) / 128 + ndocs + total_tokens / s_len), (unsigned)nk);
     if (d == 128) {
         hipLaunchKernelGGL(attn_delta_kernel<128>, dim3((unsigned)g), dim3(kThreads), 0, st, p);
         hipLaunchKernelGGL(attn_bwd_dkdv_kernel<128>, gridk, dim3(kThreads), 0, st, p);
