@@ -173,6 +173,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
     TL::load(vbase, p.v_ss, 0, doc_len, tid, rv);
     TL::store(smem, tid, rk);
     TL::store(smem + TL::ELEMS, tid, rv);
+    // every load issued so far (the per-lane operand rows included) has landed before the loop starts;
+    // otherwise their first use inside the loop would also wait for the tile loads issued just before it
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     if (ntiles > 1) {
         TL::load(kbase, p.k_ss, 64, doc_len, tid, rk);
         TL::load(vbase, p.v_ss, 64, doc_len, tid, rv);
@@ -201,24 +204,53 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
         }
         const int key0 = t * 64;
         if (key0 <= qw0 + 31) {  // otherwise every key of the tile is after every query of this wave
+            // S^T = K Q^T in groups of 4 MFMAs; the K fragments of the next group are in flight meanwhile
+            constexpr int KG = D / 64, NG = 2 * KG;
             f32x16 sacc[2];
+            bf16x8 fk[2][4];
+            auto ldk = [&](int g, int buf) {
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+                for (int i = 0; i < 4; ++i) fk[buf][i] = TL::frag_kc(sK, (g / KG) * 32, (g % KG) * 4 + i, lane);
+            };
+            ldk(0, 0);
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
 #pragma unroll
-                for (int kd = 0; kd < D / 16; ++kd)
-                    sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_kc(sK, kb * 32, kd, lane), qf[kd], sacc[kb], 0, 0, 0);
+            for (int g = 0; g < NG; ++g) {
+                if (g + 1 < NG) ldk(g + 1, (g + 1) & 1);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    sacc[g / KG] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk[g & 1][i], qf[(g % KG) * 4 + i], sacc[g / KG], 0, 0, 0);
             }
-            const bool need_mask = key0 + 63 > qw0;
+            // keep that order: the reads of group g+1 are issued before the MFMAs of group g
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                if (g + 1 < NG) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // first V^T fragments: their LDS latency hides under the softmax arithmetic
+            bf16x8 fv[2][D / 32];
+            auto ldv = [&](int g, int buf) {
+#pragma unroll
+                for (int db = 0; db < D / 32; ++db) fv[buf][db] = TL::frag_tr(sV, (g >> 1) * 32 + 16 * (g & 1), db * 32, lane);
+            };
+            ldv(0, 0);
+            if (key0 + 63 > qw0) {  // the tile touches the diagonal: mask keys after the query
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (key0 + kb * 32 + acc_row(r, lane) > qi) sacc[kb][r] = -INFINITY;
+            }
             float mloc = -INFINITY;  // running maximum is kept on the raw (unscaled) scores
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    if (need_mask && key0 + kb * 32 + acc_row(r, lane) > qi) sacc[kb][r] = -INFINITY;
-                    mloc = fmaxf(mloc, sacc[kb][r]);
-                }
+                for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, sacc[kb][r]);
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
             const float mnew = fmaxf(m, mloc);
             const float moff = (mnew == -INFINITY ? 0.f : mnew) * sl2;
@@ -241,16 +273,15 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
             }
             lsum += psum;
             m = mnew;
+            // O^T += V^T P^T, 4 groups of (16 keys x all d blocks)
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int g = 0; g < 4; ++g) {
+                if (g + 1 < 4) ldv(g + 1, (g + 1) & 1);
+                const bf16x8 pf = acc_to_b(sacc[g >> 1], g & 1);
 #pragma unroll
-                for (int tt = 0; tt < 2; ++tt) {
-                    const bf16x8 pf = acc_to_b(sacc[kb], tt);
-#pragma unroll
-                    for (int db = 0; db < D / 32; ++db)
-                        oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_tr(sV, kb * 32 + 16 * tt, db * 32, lane), pf,
-                                                                           oacc[db], 0, 0, 0);
-                }
+                for (int db = 0; db < D / 32; ++db)
+                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv[g & 1][db], pf, oacc[db], 0, 0, 0);
+            }
         }
         __syncthreads();
     }
@@ -348,6 +379,7 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
     };
     load_iter(0);
     store_iter(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K/V rows held in registers have landed (see the forward kernel)
     if (total > 1) load_iter(1);
     __syncthreads();
 
@@ -362,14 +394,47 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
         for (int sub = 0; sub < 2; ++sub) {
             const int qs0 = qbase + sub * 32;
             if (qs0 + 31 < kw0 || qs0 >= doc_len) continue;  // all queries before this wave's keys / past the end
+            // S = Q K^T and dP = dO V^T in groups of 2 d-steps; the next group's fragments are in flight meanwhile
+            constexpr int NG = D / 32;
             f32x16 sacc, dpacc;
+            bf16x8 fq[2][2], fo[2][2];
+            auto ldqo = [&](int g, int buf) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    fq[buf][i] = TL::frag_kc(sQ, sub * 32, g * 2 + i, lane);
+                    fo[buf][i] = TL::frag_kc(sdO, sub * 32, g * 2 + i, lane);
+                }
+            };
+            ldqo(0, 0);
 #pragma unroll
             for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
 #pragma unroll
-            for (int kd = 0; kd < D / 16; ++kd) {
-                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_kc(sQ, sub * 32, kd, lane), kf[kd], sacc, 0, 0, 0);
-                dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_kc(sdO, sub * 32, kd, lane), vf[kd], dpacc, 0, 0, 0);
+            for (int g = 0; g < NG; ++g) {
+                if (g + 1 < NG) ldqo(g + 1, (g + 1) & 1);
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[g & 1][i], kf[g * 2 + i], sacc, 0, 0, 0);
+                    dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fo[g & 1][i], vf[g * 2 + i], dpacc, 0, 0, 0);
+                }
             }
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                if (g + 1 < NG) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+            }
+            // dO^T / Q^T fragments, two d blocks at a time; the first pair's latency hides under the elementwise math
+            constexpr int NT = 2 * (D / 64);  // (16-query step, d-block pair) groups
+            bf16x8 fto[2][2], ftq[2][2];
+            auto ldt = [&](int gt, int buf) {
+                const int tt = gt / (D / 64), dbp = gt % (D / 64);
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    fto[buf][i] = TL::frag_tr(sdO, sub * 32 + 16 * tt, (2 * dbp + i) * 32, lane);
+                    ftq[buf][i] = TL::frag_tr(sQ, sub * 32 + 16 * tt, (2 * dbp + i) * 32, lane);
+                }
+            };
+            ldt(0, 0);
             // accumulator register r <-> query qs0 + acc_row(r); lane <-> key kj
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
@@ -387,15 +452,15 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
                 }
             }
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
+            for (int gt = 0; gt < NT; ++gt) {
+                if (gt + 1 < NT) ldt(gt + 1, (gt + 1) & 1);
+                const int tt = gt / (D / 64), dbp = gt % (D / 64);
                 const bf16x8 pf = acc_to_b(sacc, tt);
                 const bf16x8 dsf = acc_to_b(dpacc, tt);
 #pragma unroll
-                for (int db = 0; db < D / 32; ++db) {
-                    dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_tr(sdO, sub * 32 + 16 * tt, db * 32, lane), pf,
-                                                                        dvacc[db], 0, 0, 0);
-                    dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_tr(sQ, sub * 32 + 16 * tt, db * 32, lane), dsf,
-                                                                        dkacc[db], 0, 0, 0);
+                for (int i = 0; i < 2; ++i) {
+                    dvacc[2 * dbp + i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fto[gt & 1][i], pf, dvacc[2 * dbp + i], 0, 0, 0);
+                    dkacc[2 * dbp + i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ftq[gt & 1][i], dsf, dkacc[2 * dbp + i], 0, 0, 0);
                 }
             }
         }
@@ -453,6 +518,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
     TL::load(vbase, p.v_ss, 0, doc_len, tid, rv);
     TL::store(smem, tid, rk);
     TL::store(smem + TL::ELEMS, tid, rv);
+    // every load issued so far (the per-lane operand rows included) has landed before the loop starts;
+    // otherwise their first use inside the loop would also wait for the tile loads issued just before it
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     if (ntiles > 1) {
         TL::load(kbase, p.k_ss, 64, doc_len, tid, rk);
         TL::load(vbase, p.v_ss, 64, doc_len, tid, rv);
@@ -480,29 +548,59 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
         }
         const int key0 = t * 64;
         if (key0 <= qw0 + 31) {
+            const bool on_diag = key0 + 63 > qw0;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
+                // S^T = K Q^T and dP^T = V dO^T in groups of 2 d-steps with the next group's fragments in flight
+                constexpr int NG = D / 32;
                 f32x16 sacc, dpacc;
+                bf16x8 fk[2][2], fvv[2][2];
+                auto ldkv = [&](int g, int buf) {
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        fk[buf][i] = TL::frag_kc(sK, kb * 32, g * 2 + i, lane);
+                        fvv[buf][i] = TL::frag_kc(sV, kb * 32, g * 2 + i, lane);
+                    }
+                };
+                ldkv(0, 0);
 #pragma unroll
                 for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
 #pragma unroll
-                for (int kd = 0; kd < D / 16; ++kd) {
-                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_kc(sK, kb * 32, kd, lane), qf[kd], sacc, 0, 0, 0);
-                    dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_kc(sV, kb * 32, kd, lane), dof[kd], dpacc, 0, 0, 0);
+                for (int g = 0; g < NG; ++g) {
+                    if (g + 1 < NG) ldkv(g + 1, (g + 1) & 1);
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk[g & 1][i], qf[g * 2 + i], sacc, 0, 0, 0);
+                        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fvv[g & 1][i], dof[g * 2 + i], dpacc, 0, 0, 0);
+                    }
                 }
+                __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+                for (int g = 0; g < NG; ++g) {
+                    if (g + 1 < NG) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                // K^T fragments of the first 16 keys: issued before the elementwise math
+                bf16x8 ftk[2][D / 32];
+                auto ldt = [&](int tt, int buf) {
+#pragma unroll
+                    for (int db = 0; db < D / 32; ++db) ftk[buf][db] = TL::frag_tr(sK, kb * 32 + 16 * tt, db * 32, lane);
+                };
+                ldt(0, 0);
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    float pe = __builtin_amdgcn_exp2f(sacc[r] * sl2 - lse2);
-                    if (key0 + kb * 32 + acc_row(r, lane) > qi) pe = 0.f;
+                    float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], sl2, -lse2));
+                    if (on_diag && key0 + kb * 32 + acc_row(r, lane) > qi) pe = 0.f;
                     dpacc[r] = pe * (dpacc[r] - dlt);
                 }
 #pragma unroll
                 for (int tt = 0; tt < 2; ++tt) {
+                    if (tt == 0) ldt(1, 1);
                     const bf16x8 dsf = acc_to_b(dpacc, tt);
 #pragma unroll
                     for (int db = 0; db < D / 32; ++db)
-                        dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(TL::frag_tr(sK, kb * 32 + 16 * tt, db * 32, lane), dsf,
-                                                                            dqacc[db], 0, 0, 0);
+                        dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ftk[tt][db], dsf, dqacc[db], 0, 0, 0);
                 }
             }
         }
