@@ -130,20 +130,67 @@ __global__ __launch_bounds__(kBlock) void embed_gather_kernel(const int64_t* __r
     }
 }
 
-// dW[ids[r], :] += dY[r, :] in fp32 (hardware float atomics: summation order is not fixed)
-__global__ __launch_bounds__(kBlock) void embed_scatter_add_kernel(const int64_t* __restrict__ ids,
-                                                                   const bf16_t* __restrict__ dY, float* __restrict__ dW,
-                                                                   int64_t rows, int h, int64_t V) {
+// dW[id, :] += sum of dY[r, :] over all rows r with ids[r] == id, without atomics and in a fixed order:
+// the block of the FIRST row holding an id owns that id; it scans the later rows 256 at a time and adds the
+// (rare) duplicates in increasing row order, then does one read-modify-write of the fp32 row.
+template <int MAXC>
+__global__ __launch_bounds__(kBlock) void embed_scatter_owner_kernel(const int64_t* __restrict__ ids, const bf16_t* __restrict__ dY,
+                                                                     float* __restrict__ dW, int64_t rows, int h, int64_t V) {
+    __shared__ unsigned long long bits[kBlock / 64];
     const int h8 = h >> 3;
-    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
-        const int64_t id = ids[r];
+    for (int64_t t = blockIdx.x; t < rows; t += gridDim.x) {
+        const int64_t id = ids[t];
         if (id < 0 || id >= V) continue;
-        for (int c = threadIdx.x; c < h8; c += kBlock) {
-            float g[8];
-            unpack8(ld_bf16x8(dY + r * h + c * 8), g);
-            float* dst = dW + id * h + c * 8;
+        int earlier = 0;
+        for (int64_t j = threadIdx.x; j < t; j += kBlock) earlier |= (ids[j] == id);
+        if (__syncthreads_or(earlier)) continue;  // an earlier row owns this id
+        float acc[MAXC][8];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) atomicAdd(dst + k, g[k]);
+        for (int c = 0; c < MAXC; ++c) {
+            const int col = (c * kBlock + threadIdx.x);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) acc[c][k] = 0.f;
+            if (col < h8) unpack8(ld_bf16x8(dY + t * h + col * 8), acc[c]);
+        }
+        for (int64_t base = t + 1; base < rows; base += kBlock) {
+            const int64_t j = base + threadIdx.x;
+            const int match = (j < rows) && (ids[j] == id);
+            if (__syncthreads_or(match)) {
+                const unsigned long long b = __ballot(match);
+                if ((threadIdx.x & 63) == 0) bits[threadIdx.x >> 6] = b;
+                __syncthreads();
+                for (int wv = 0; wv < kBlock / 64; ++wv) {
+                    unsigned long long m = bits[wv];
+                    while (m) {
+                        const int l = __builtin_ctzll(m);
+                        m &= m - 1;
+                        const int64_t jj = base + wv * 64 + l;
+#pragma unroll
+                        for (int c = 0; c < MAXC; ++c) {
+                            const int col = (c * kBlock + threadIdx.x);
+                            if (col < h8) {
+                                float g[8];
+                                unpack8(ld_bf16x8(dY + jj * h + col * 8), g);
+#pragma unroll
+                                for (int k = 0; k < 8; ++k) acc[c][k] += g[k];
+                            }
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < MAXC; ++c) {
+            const int col = (c * kBlock + threadIdx.x);
+            if (col < h8) {
+                float* dst = dW + id * h + col * 8;
+                f32x4 lo = *reinterpret_cast<f32x4*>(dst), hi = *reinterpret_cast<f32x4*>(dst + 4);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) { lo[k] += acc[c][k]; hi[k] += acc[c][4 + k]; }
+                *reinterpret_cast<f32x4*>(dst) = lo;
+                *reinterpret_cast<f32x4*>(dst + 4) = hi;
+            }
         }
     }
 }
@@ -300,8 +347,17 @@ extern "C" int ezl_embed_scatter_add(const void* ids, const void* dy, void* dwei
     EZL_REQUIRE((rows == 0 || (ids && dy && dweight_f32)) && ezl_aligned16(dy), EZL_EINVAL,
                 "ezl_embed_scatter_add: null or misaligned pointer");
     if (rows == 0) return EZL_OK;
-    hipLaunchKernelGGL(embed_scatter_add_kernel, dim3(grid_for(rows, 1)), dim3(kBlock), 0, (hipStream_t)stream,
-                       (const int64_t*)ids, (const bf16_t*)dy, (float*)dweight_f32, rows, (int)h, vocab);
+    EZL_REQUIRE(h <= 8192 * 2, EZL_EUNSUPPORTED, "ezl_embed_scatter_add: h must be <= 16384");
+    EZL_REQUIRE(((uintptr_t)dweight_f32 & 15) == 0, EZL_EINVAL, "ezl_embed_scatter_add: dweight must be 16-byte aligned");
+    if (h <= 8 * kBlock * 2)
+        hipLaunchKernelGGL((embed_scatter_owner_kernel<2>), dim3(grid_for(rows, 1)), dim3(kBlock), 0, (hipStream_t)stream,
+                           (const int64_t*)ids, (const bf16_t*)dy, (float*)dweight_f32, rows, (int)h, vocab);
+    else if (h <= 8 * kBlock * 4)
+        hipLaunchKernelGGL((embed_scatter_owner_kernel<4>), dim3(grid_for(rows, 1)), dim3(kBlock), 0, (hipStream_t)stream,
+                           (const int64_t*)ids, (const bf16_t*)dy, (float*)dweight_f32, rows, (int)h, vocab);
+    else
+        hipLaunchKernelGGL((embed_scatter_owner_kernel<8>), dim3(grid_for(rows, 1)), dim3(kBlock), 0, (hipStream_t)stream,
+                           (const int64_t*)ids, (const bf16_t*)dy, (float*)dweight_f32, rows, (int)h, vocab);
     EZL_LAUNCH_CHECK("ezl_embed_scatter_add");
     return EZL_OK;
 }

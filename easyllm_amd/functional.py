@@ -60,6 +60,46 @@ def linear(x, weight):
     return LinearFunction.apply(x, weight)
 
 
+class FanOutLinearFunction(torch.autograd.Function):
+    """One input through several bias-free linears (q/k/v, or gate/up): y_i = x W_i^T.  The input gradient
+    sum_i dy_i W_i is accumulated inside the GEMM epilogue instead of by separate add kernels."""
+
+    @staticmethod
+    def forward(ctx, x, *weights):
+        x2d = x.reshape(-1, x.shape[-1])
+        ctx.save_for_backward(x, *weights)
+        return tuple(K.linear_fwd(x2d, w).view(*x.shape[:-1], w.shape[0]) for w in weights)
+
+    @staticmethod
+    def backward(ctx, *dys):
+        x, *weights = ctx.saved_tensors
+        x2d = x.reshape(-1, x.shape[-1])
+        dx = None
+        grads = []
+        for i, (dy, w) in enumerate(zip(dys, weights)):
+            if dy is None:
+                grads.append(None)
+                continue
+            dy2d = dy.reshape(-1, dy.shape[-1])
+            if not dy2d.is_contiguous():
+                dy2d = dy2d.contiguous()
+            if ctx.needs_input_grad[0]:
+                dx = K.linear_dgrad(dy2d, w, out=dx, accumulate=dx is not None)
+            dw = None
+            if ctx.needs_input_grad[1 + i]:
+                mg, acc = _main_grad_target(w)
+                if mg is not None:
+                    K.linear_wgrad(dy2d, x2d, out=mg, accumulate=acc)
+                else:
+                    dw = K.linear_wgrad(dy2d, x2d)
+            grads.append(dw)
+        return (None if dx is None else dx.view(x.shape),) + tuple(grads)
+
+
+def fan_out_linear(x, *weights):
+    return FanOutLinearFunction.apply(x, *weights)
+
+
 class BiasAddFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, bias):
@@ -113,8 +153,32 @@ class AddRMSNormFunction(torch.autograd.Function):
         return dx, dx, dw, None
 
 
+class RMSNormPassFunction(torch.autograd.Function):
+    """x -> (x, rmsnorm(x) * w): the pre-norm block keeps x as its residual, so the gradient arriving on the
+    residual branch is added inside the norm's backward kernel instead of by a separate add."""
+
+    @staticmethod
+    def forward(ctx, x, weight, eps):
+        xc = x.contiguous()
+        y, rstd, _ = K.rmsnorm_fwd(xc, weight, eps)
+        ctx.save_for_backward(xc, weight, rstd)
+        return xc.view_as(xc), y
+
+    @staticmethod
+    def backward(ctx, dres, dy):
+        x, weight, rstd = ctx.saved_tensors
+        mg, acc = _main_grad_target(weight)
+        dx, dw = K.rmsnorm_bwd(dy.contiguous(), x, weight, rstd, dresidual=None if dres is None else dres.contiguous(),
+                               main_grad=mg, accumulate=acc)
+        return dx, dw, None
+
+
 def rmsnorm(x, weight, eps):
     return RMSNormFunction.apply(x, weight, eps)
+
+
+def rmsnorm_pass(x, weight, eps):
+    return RMSNormPassFunction.apply(x, weight, eps)
 
 
 def add_rmsnorm(x, residual, weight, eps):

@@ -211,11 +211,11 @@ def linear_fwd(x2d, w):
     return gemm(x2d, w, x2d.shape[0], w.shape[0], x2d.shape[1], lda, ldb, True, True)
 
 
-def linear_dgrad(dy2d, w):
-    """dx[T, in] = dy[T, out] @ w[out, in]"""
+def linear_dgrad(dy2d, w, out=None, accumulate=False):
+    """dx[T, in] (=|+=) dy[T, out] @ w[out, in]"""
     lda, ldb = _rows_ld(dy2d, "dy"), _rows_ld(w, "w")
     _need(dy2d.shape[1] == w.shape[0], "linear_dgrad: inner dimensions differ")
-    return gemm(dy2d, w, dy2d.shape[0], w.shape[1], w.shape[0], lda, ldb, True, False)
+    return gemm(dy2d, w, dy2d.shape[0], w.shape[1], w.shape[0], lda, ldb, True, False, out=out, accumulate=accumulate)
 
 
 def linear_wgrad(dy2d, x2d, out=None, accumulate=False):

@@ -109,6 +109,13 @@ class RMSNorm(torch.nn.Module):
         _require_bf16(input, "RMSNorm")
         return F_.rmsnorm(input, self.weight, self.eps)
 
+    def forward_keep_input(self, x):
+        """(x, norm(x)): x is returned as the residual branch so that its gradient is fused into the norm's backward."""
+        if self.layernorm_tp_auto_sync or self.sequence_parallel:
+            dist_env.sync_tp_duplicated_parameter(self.weight)
+        _require_bf16(x, "RMSNorm")
+        return F_.rmsnorm_pass(x, self.weight, self.eps)
+
     def forward_with_residual(self, x, residual):
         """(x + residual, norm(x + residual)) in one kernel -- transformer.py:786-787 fused."""
         if self.layernorm_tp_auto_sync or self.sequence_parallel:

@@ -81,8 +81,8 @@ class ParallelMLP(torch.nn.Module):
                                            sequence_parallel=sequence_parallel)
 
     def forward(self, hidden_states):
-        h1, _ = self.gate_proj(hidden_states)
-        h2, _ = self.up_proj(hidden_states)
+        # gate_proj and up_proj share their input: one fan-out op (input gradient accumulated in the GEMM)
+        h1, h2 = F_.fan_out_linear(hidden_states, self.gate_proj.weight, self.up_proj.weight)
         h1 = self.activation_func.fused_mul(h1, h2)
         return self.down_proj(h1)
 
@@ -157,7 +157,10 @@ class ParallelAttention(torch.nn.Module):
         # hidden_states [s, b, h]
         if layer_past is not None or get_key_value:
             raise NotImplementedError("KV-cache inference is outside the training step")
-        if not self.qkv_pack:
+        if not self.qkv_pack and self.q_proj.bias is None:
+            query_layer, key_layer, value_layer = F_.fan_out_linear(hidden_states, self.q_proj.weight, self.k_proj.weight,
+                                                                    self.v_proj.weight)
+        elif not self.qkv_pack:
             query_layer, _ = self.q_proj(hidden_states)
             key_layer, _ = self.k_proj(hidden_states)
             value_layer, _ = self.v_proj(hidden_states)
@@ -235,7 +238,7 @@ class ParallelTransformerLayer(torch.nn.Module):
 
     def forward(self, hidden_states, attention_mask, cu_seqlens=None, position_ids=None, layer_past=None,
                 get_key_value=False):
-        layernorm_output = self.input_layernorm(hidden_states)
+        hidden_states, layernorm_output = self.input_layernorm.forward_keep_input(hidden_states)
         attention_output, attention_bias = self.self_attn(layernorm_output, attention_mask, cu_seqlens, position_ids,
                                                           layer_past=layer_past, get_key_value=get_key_value, alibi=self.alibi)
         if attention_bias is not None:

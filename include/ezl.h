@@ -58,7 +58,7 @@ int ezl_rope_apply(const void* x, void* out, const void* cos_table, const void* 
 /* ---- token embedding: base_modules/layers/vocab_parallel_emb.py:106-137 (F.embedding, TP=1) ----
  * gather: out[r] = weight[ids[r]] (bit-exact row copy); an id outside [0, vocab) ORs 1 (id >= vocab)
  * or 2 (id < 0) into *bad_flag (device int32) and yields a zero row.
- * scatter_add: dweight_f32[ids[r]] += dy[r] with fp32 atomics (summation order not fixed). */
+ * scatter_add: dweight_f32[id] += sum of dy[r] over rows with ids[r] == id, fp32, no atomics, fixed (row) order. */
 int ezl_embed_gather(const void* ids, const void* weight, void* out, void* bad_flag, int64_t rows, int64_t h, int64_t vocab,
                      void* stream);
 int ezl_embed_scatter_add(const void* ids, const void* dy, void* dweight_f32, int64_t rows, int64_t h, int64_t vocab,

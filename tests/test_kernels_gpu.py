@@ -127,14 +127,28 @@ def test_embedding_gather_exact_and_flag(K, gpu_device):
         O.embedding(bad, W)
 
 
-def test_embedding_scatter_add(K, gpu_device):
-    V, h = 50, 64
-    ids = torch.randint(0, V, (3, 200), generator=torch.Generator().manual_seed(3))
-    dy = rnd(3, 200, h, seed=10)
-    dW = torch.zeros(V, h, dtype=torch.float32, device=gpu_device)
+@pytest.mark.parametrize("V,h,shape", [(50, 64, (3, 200)), (7, 4096, (1, 700)), (300, 8200, (2, 150))])
+def test_embedding_scatter_add(K, gpu_device, V, h, shape):
+    """Heavy id collisions (V << rows); the sum per id runs in row order in fp32, so the result is bit-exact
+    against a sequential fp32 loop, adds onto what the buffer already holds, and repeats identically."""
+    print("embed scatter", V, h, shape, flush=True)
+    ids = torch.randint(0, V, shape, generator=torch.Generator().manual_seed(3))
+    dy = rnd(*shape, h, seed=10)
+    init = torch.randn(V, h, generator=torch.Generator().manual_seed(4))
+    dW = init.to(gpu_device)
     K.embed_scatter_add(ids.to(gpu_device), dy.to(gpu_device), dW)
     ref = O.embedding_bwd(ids, dy.float(), V)
-    assert torch.allclose(dW.cpu(), ref, rtol=1e-5, atol=1e-5)  # fp32 sums, order differs only
+    assert torch.allclose(dW.cpu() - init, ref, rtol=1e-4, atol=1e-4)
+    seq = torch.zeros(V, h)
+    seen = set()
+    flat_ids, flat_dy = ids.reshape(-1).tolist(), dy.float().reshape(-1, h)
+    for r, i in enumerate(flat_ids):  # first occurrence starts the sum, later rows add in order
+        seq[i] = flat_dy[r] if i not in seen else seq[i] + flat_dy[r]
+        seen.add(i)
+    assert torch.equal(dW.cpu(), init + seq)
+    dW2 = init.to(gpu_device)
+    K.embed_scatter_add(ids.to(gpu_device), dy.to(gpu_device), dW2)
+    assert torch.equal(dW2, dW)
 
 
 # ------------------------------------------------------------------------------------- plumbing
