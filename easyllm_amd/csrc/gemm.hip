@@ -228,35 +228,49 @@ typedef __attribute__((address_space(1))) const void gvoid;
 // One operand tile = 32 wave-instructions of 1 KiB each (global_load_lds_dwordx4: lane l lands at base + 16 l).
 //   k-contiguous tile [256 rows][64 k]:  instruction q covers rows 8q..8q+7; chunk c of row r sits in slot c ^ ((r>>1)&7)
 //   k-major tile      [64 k][256 cols]:  instruction q covers k rows 2q, 2q+1; chunk c of k row sits in slot c ^ ((k&3)<<2)
+// Wave w issues instructions q = w*NI .. w*NI+NI-1, i.e. one contiguous NI KiB piece of the tile: M0 (the LDS base) is
+// written once per tile and the instruction offset i*1024 selects the KiB.  That offset is also added to the global
+// address, so the per-lane byte offsets are stored with i*1024 already subtracted; they are kept 4 KiB high (and the scalar
+// base 4 KiB low) so that they stay non-negative.  The address is scalar base + 32-bit lane offset + immediate: no vector
+// address arithmetic inside the K loop.
 template <bool KC, int NW>
 struct Loader {
     static constexpr int NI = 32 / NW;
-    uint32_t off[NI];
+    static_assert(NI * 1024 <= 4096, "instruction offsets are limited to 12 bits");
+    uint32_t off[NI];  // byte offsets from (operand base + k advance - 4096)
     __device__ __forceinline__ void init(int lane, int wave, int first, int dim, int64_t ld) {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int q = wave + NW * i;
+            const int q = wave * NI + i;
+            int64_t e;
             if (KC) {
                 const int row = 8 * q + (lane >> 3);
                 const int c = (lane & 7) ^ ((row >> 1) & 7);
                 int gr = first + row;
                 gr = gr < dim ? gr : dim - 1;
-                off[i] = (uint32_t)((int64_t)gr * ld + c * 8);
+                e = (int64_t)gr * ld + c * 8;
             } else {
                 const int krow = 2 * q + (lane >> 5);
                 const int c = (lane & 31) ^ ((krow & 3) << 2);
                 int col = first + c * 8;
                 col = col + 8 <= dim ? col : dim - 8;
-                off[i] = (uint32_t)((int64_t)krow * ld + col);
+                e = (int64_t)krow * ld + col;
             }
+            off[i] = (uint32_t)(e * 2 + 4096 - i * 1024);
         }
     }
-    __device__ __forceinline__ void issue(const bf16_t* __restrict__ gbase, bf16_t* stage, int wave) const {
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const int q = wave + NW * i;
-            __builtin_amdgcn_global_load_lds((gvoid*)(gbase + off[i]), (lds_void*)(stage + q * 512), 16, 0, 0);
-        }
+    // gbase: operand base advanced to the tile's first k, as a byte pointer
+    template <int I>
+    __device__ __forceinline__ void issue_one(const char* gbase, bf16_t* piece) const {
+        __builtin_amdgcn_global_load_lds((gvoid*)(gbase - 4096 + off[I]), (lds_void*)piece, 16, I * 1024, 0);
+    }
+    __device__ __forceinline__ void issue(const bf16_t* __restrict__ gtile, bf16_t* stage, int wave) const {
+        const char* gbase = reinterpret_cast<const char*>(gtile);
+        bf16_t* piece = stage + wave * (NI * 512);
+        issue_one<0>(gbase, piece);
+        if constexpr (NI > 1) issue_one<1>(gbase, piece);
+        if constexpr (NI > 2) issue_one<2>(gbase, piece);
+        if constexpr (NI > 3) issue_one<3>(gbase, piece);
     }
 };
 
@@ -280,6 +294,39 @@ __device__ __forceinline__ bf16x8 sfrag(const bf16_t* __restrict__ s, int row0, 
         return v;
     }
 }
+
+// Instruction-scheduling recipes (compile-time unrolled): one MFMA, then up to PER LDS reads, ... until the reads run out.
+template <int MASK, int N>
+__device__ __forceinline__ void sched_group() {
+    if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
+}
+template <int G, int NM, int RD, int PER>
+struct SchedInner {
+    static __device__ __forceinline__ void run() {
+        if constexpr (G < NM) {
+            sched_group<SG_MFMA, 1>();
+            constexpr int left = RD - G * PER;
+            sched_group<SG_DS_R, (left > PER ? PER : (left > 0 ? left : 0))>();
+            SchedInner<G + 1, NM, RD, PER>::run();
+        }
+    }
+};
+// ... and for the sub-step behind the barrier: LDS reads first, global->LDS loads in the MFMA slots after them
+template <int G, int NM, int RD, int PER, int NLD, int PER_V>
+struct SchedLast {
+    static __device__ __forceinline__ void run() {
+        if constexpr (G < NM) {
+            sched_group<SG_MFMA, 1>();
+            constexpr int left = RD - G * PER;
+            constexpr int nds = left > PER ? PER : (left > 0 ? left : 0);
+            constexpr int ds_slots = PER > 0 ? (RD + PER - 1) / PER : 0;
+            constexpr int vleft = G >= ds_slots ? NLD - (G - ds_slots) * PER_V : 0;
+            sched_group<SG_DS_R, nds>();
+            sched_group<SG_VMEM_R, (vleft > PER_V ? PER_V : (vleft > 0 ? vleft : 0))>();
+            SchedLast<G + 1, NM, RD, PER, NLD, PER_V>::run();
+        }
+    }
+};
 
 template <bool A_KC, bool B_KC, typename OutT, int WAVES_M, int WAVES_N>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_d2l_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
@@ -327,12 +374,14 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_d2l_kernel(const 
     const int64_t bstep = B_KC ? BK : (int64_t)BK * ldb;
     const int arow = wm * (TM * 32), brow = wn * (TN * 32);
 
+    // Fragment reads go B first, then A: the first MFMAs of a sub-step need both B fragments and A[0] only, and LDS returns
+    // data in issue order, so the waits in front of those MFMAs cover the oldest reads instead of all of them.
     bf16x8 fa[2][TM], fb[2][TN];
     auto read_frags = [&](const bf16_t* sA, int ks, int buf) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[buf][i] = sfrag<A_KC>(sA, arow + i * 32, ks, lane);
-#pragma unroll
         for (int j = 0; j < TN; ++j) fb[buf][j] = sfrag<B_KC>(sA + DTILE, brow + j * 32, ks, lane);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[buf][i] = sfrag<A_KC>(sA, arow + i * 32, ks, lane);
     };
     auto mfmas = [&](int buf) {
 #pragma unroll
@@ -348,11 +397,26 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_d2l_kernel(const 
 
     issue_tile(0, 0);
     if (nk > 1) issue_tile(1, 1);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    // Pull the remaining kernel arguments into registers now: a scalar load still in flight inside the K loop shares the
+    // counter of the LDS reads and would turn every counted wait on them into a full drain.
+    asm volatile("" ::"s"(C), "s"(ldc), "s"(accumulate));
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
     __syncthreads();
     read_frags(smem, 0, 0);
 
     constexpr int RD = (A_KC ? TM : 2 * TM) + (B_KC ? TN : 2 * TN);  // LDS reads per sub-step
+    constexpr int NM = TM * TN;                                      // MFMAs per sub-step
+    constexpr int NLD = 2 * (32 / NW);                               // global->LDS loads per wave and tile pair
+    // inner sub-steps: the reads of the next sub-step are issued behind the first MFMAs, leaving the last two MFMAs as slack
+#ifndef EZL_PER_MIN
+#define EZL_PER_MIN 1
+#endif
+    constexpr int PER0 = (RD + NM - 3) / (NM - 2);
+    constexpr int PER = PER0 > EZL_PER_MIN ? PER0 : EZL_PER_MIN;
+    // last sub-step: reads of the next tile's first fragments first, then the loads of tile kt+2
+    constexpr int PER_L = (RD + NM / 2 - 1) / (NM / 2);
+    constexpr int DS_SLOTS_L = (RD + PER_L - 1) / PER_L;
+    constexpr int PER_V = (NLD + (NM - DS_SLOTS_L) - 1) / (NM - DS_SLOTS_L);
 #define EZL_STEP(HAS_NEXT, DO_LOAD)                                                                       \
     {                                                                                                     \
         const int cur = kt & 1;                                                                           \
@@ -360,23 +424,16 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_d2l_kernel(const 
         _Pragma("unroll") for (int ks = 0; ks < NKS - 1; ++ks) {                                          \
             read_frags(sA, ks + 1, (ks + 1) & 1);                                                         \
             mfmas(ks & 1);                                                                                \
-            _Pragma("unroll") for (int g = 0; g < TM * TN / 2; ++g) {                                     \
-                __builtin_amdgcn_sched_group_barrier(SG_MFMA, 2, 0);                                      \
-                __builtin_amdgcn_sched_group_barrier(SG_DS_R, RD > TM * TN / 2 ? 2 : 1, 0);               \
-            }                                                                                             \
+            SchedInner<0, NM, RD, PER>::run();                                                            \
         }                                                                                                 \
         __builtin_amdgcn_sched_barrier(0);                                                                \
         __builtin_amdgcn_s_waitcnt(0x0F70);                                                               \
         __syncthreads();                                                                                  \
         __builtin_amdgcn_sched_barrier(0);                                                                \
-        if (DO_LOAD) issue_tile(kt + 2, cur);                                                             \
         if (HAS_NEXT) read_frags(smem + (cur ^ 1) * 2 * DTILE, 0, 0);                                      \
+        if (DO_LOAD) issue_tile(kt + 2, cur);                                                             \
         mfmas((NKS - 1) & 1);                                                                             \
-        _Pragma("unroll") for (int g = 0; g < TM * TN / 2; ++g) {                                         \
-            __builtin_amdgcn_sched_group_barrier(SG_MFMA, 2, 0);                                          \
-            if (DO_LOAD) __builtin_amdgcn_sched_group_barrier(SG_VMEM_R, 2, 0);                           \
-            if (HAS_NEXT) __builtin_amdgcn_sched_group_barrier(SG_DS_R, RD > TM * TN / 2 ? 2 : 1, 0);     \
-        }                                                                                                 \
+        SchedLast<0, NM, (HAS_NEXT) ? RD : 0, PER_L, (DO_LOAD) ? NLD : 0, PER_V>::run();                  \
         __builtin_amdgcn_sched_barrier(0);                                                                \
     }
 
@@ -437,8 +494,8 @@ extern "C" int ezl_gemm_bf16(const void* A, const void* B, void* C, int64_t M, i
     EZL_REQUIRE(b_kc ? (K % 8 == 0) : (N % 8 == 0), EZL_EUNSUPPORTED, "ezl_gemm_bf16: contiguous extent of B must be a multiple of 8");
     EZL_REQUIRE(lda >= (a_kc ? K : M) && ldb >= (b_kc ? K : N) && ldc >= N, EZL_EINVAL, "ezl_gemm_bf16: leading dimension too small");
     const int64_t a_rows = a_kc ? M : K, b_rows = b_kc ? N : K;
-    EZL_REQUIRE(a_rows * lda < (1LL << 32) && b_rows * ldb < (1LL << 32) && M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31),
-                EZL_EUNSUPPORTED, "ezl_gemm_bf16: operand larger than 2^32 elements");
+    EZL_REQUIRE(a_rows * lda < (1LL << 31) - 4096 && b_rows * ldb < (1LL << 31) - 4096 && M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31),
+                EZL_EUNSUPPORTED, "ezl_gemm_bf16: operand larger than 2^31 elements");
     const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     EZL_REQUIRE(tiles < (1LL << 31), EZL_EUNSUPPORTED, "ezl_gemm_bf16: too many tiles");
     hipStream_t st = (hipStream_t)stream;
