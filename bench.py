@@ -62,6 +62,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="C2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--input-check", choices=("sync", "deferred"), default="deferred",
+                    help="token-id range check of the embedding: blocking like the reference, or examined one call late")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share only (TP=1, one MI355X); --gpus %d is not supported. "
@@ -69,7 +71,7 @@ def main():
         sys.exit(2)
 
     import torch
-    from easyllm_amd import kernels, runner, workloads as W
+    from easyllm_amd import functional, kernels, runner, workloads as W
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
@@ -79,6 +81,7 @@ def main():
     torch.manual_seed(w["seed"])
     model = runner.build_model({"type": "llama_custom", "kwargs": W.model_kwargs(w)})
     runner.attach_main_grads(model)
+    functional.set_input_check(args.input_check)
     inputs, labels, doc_lens = W.make_inputs(w, device=dev)
     tokens_per_step = w["batch"] * w["seq"]
     flops = W.step_flops(w, doc_lens)
@@ -94,6 +97,7 @@ def main():
     t0 = time.perf_counter()
     for _ in range(args.steps):
         loss = step()
+    functional.flush_input_checks()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     timing, kernels.GEMM_TIMING = kernels.GEMM_TIMING, None
@@ -110,7 +114,8 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "%s: %s" % (args.workload, w["desc"]), "tokens_per_step": tokens_per_step,
-                   "fp32_main_grads": True, "recomputed_layers": model.recompute_count},
+                   "fp32_main_grads": True, "recomputed_layers": model.recompute_count,
+                   "input_id_check": args.input_check},
         "tflops": round(tflops, 1), "mfma_frac_end_to_end": round(tflops / PEAK_BF16_TFLOPS, 4), "loss": round(loss_value, 5),
         "roofline": {"kernel": "gemm_kernel (bf16 MFMA GEMM, %d launches/step)" % (len(timing) // max(args.steps, 1)),
                      "bound": "mfma", "achieved": round(gemm_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",

@@ -227,12 +227,15 @@ typedef __attribute__((address_space(1))) const void gvoid;
 
 // One operand tile = 32 wave-instructions of 1 KiB each (global_load_lds_dwordx4: lane l lands at base + 16 l).
 //   k-contiguous tile [256 rows][64 k]:  instruction q covers rows 8q..8q+7; chunk c of row r sits in slot c ^ ((r>>1)&7)
-//   k-major tile      [64 k][256 cols]:  instruction q covers k rows 2q, 2q+1; chunk c of k row sits in slot c ^ ((k&3)<<2)
+//   k-major tile      [64 k][256 cols]:  instruction q covers k rows 2q, 2q+1; chunk c of k row sits in slot c ^ kmajor_swizzle(k)
 // Wave w issues instructions q = w*NI .. w*NI+NI-1, i.e. one contiguous NI KiB piece of the tile: M0 (the LDS base) is
 // written once per tile and the instruction offset i*1024 selects the KiB.  That offset is also added to the global
 // address, so the per-lane byte offsets are stored with i*1024 already subtracted; they are kept 4 KiB high (and the scalar
 // base 4 KiB low) so that they stay non-negative.  The address is scalar base + 32-bit lane offset + immediate: no vector
 // address arithmetic inside the K loop.
+// chunk (16 B) permutation of a k-major tile row: keeps the transpose reads of one wave instruction on distinct banks
+__device__ __forceinline__ int kmajor_swizzle(int krow) { return ((krow & 3) << 2) ^ (((krow >> 3) & 1) << 1); }
+
 template <bool KC, int NW>
 struct Loader {
     static constexpr int NI = 32 / NW;
@@ -251,7 +254,7 @@ struct Loader {
                 e = (int64_t)gr * ld + c * 8;
             } else {
                 const int krow = 2 * q + (lane >> 5);
-                const int c = (lane & 31) ^ ((krow & 3) << 2);
+                const int c = (lane & 31) ^ kmajor_swizzle(krow);
                 int col = first + c * 8;
                 col = col + 8 <= dim ? col : dim - 8;
                 e = (int64_t)krow * ld + col;
@@ -274,20 +277,21 @@ struct Loader {
     }
 };
 
+// ---- LDS -> MFMA 16x16x32 operand fragment: 16 rows (or columns) x 32 k; lane l holds row l & 15, k = 8 (l >> 4) + 0..7 ----
 template <bool KC>
 __device__ __forceinline__ bf16x8 sfrag(const bf16_t* __restrict__ s, int row0, int ks, int lane) {
     if (KC) {
-        const int row = row0 + (lane & 31);
-        const int c = (ks * 2 + (lane >> 5)) ^ ((row >> 1) & 7);
+        const int row = row0 + (lane & 15);
+        const int c = (ks * 4 + (lane >> 4)) ^ ((row >> 1) & 7);
         return *reinterpret_cast<const bf16x8*>(s + row * 64 + c * 8);
     } else {
-        const int q = lane >> 4;
-        const int krow = ks * 16 + (q >> 1) * 8 + ((lane & 15) >> 2);
-        const int col = row0 + (q & 1) * 16 + ((lane & 3) << 2);
-        const int c = (col >> 3) ^ ((krow & 3) << 2);
+        // a 16-lane group reads an 8(k) x 16(row) block as two 4 x 16 transpose reads; lane i of the group receives column i
+        const int krow = ks * 32 + (lane >> 4) * 8 + ((lane & 15) >> 2);
+        const int col = row0 + ((lane & 3) << 2);
+        const int c = (col >> 3) ^ kmajor_swizzle(krow);
         const bf16_t* p = s + krow * 256 + c * 8 + (col & 7);
         const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p));
-        const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p + 4 * 256));
+        const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p + 4 * 256));  // k + 4: same swizzle
         bf16x8 v;
         v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
         v[4] = hi[0]; v[5] = hi[1]; v[6] = hi[2]; v[7] = hi[3];
@@ -295,47 +299,40 @@ __device__ __forceinline__ bf16x8 sfrag(const bf16_t* __restrict__ s, int row0, 
     }
 }
 
-// Instruction-scheduling recipes (compile-time unrolled): one MFMA, then up to PER LDS reads, ... until the reads run out.
+// Instruction-scheduling recipe for one phase (compile-time unrolled): one MFMA, then up to PER LDS reads while reads are
+// left, then up to PER_V global->LDS loads while loads are left.
 template <int MASK, int N>
 __device__ __forceinline__ void sched_group() {
     if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
 }
-template <int G, int NM, int RD, int PER>
-struct SchedInner {
-    static __device__ __forceinline__ void run() {
-        if constexpr (G < NM) {
-            sched_group<SG_MFMA, 1>();
-            constexpr int left = RD - G * PER;
-            sched_group<SG_DS_R, (left > PER ? PER : (left > 0 ? left : 0))>();
-            SchedInner<G + 1, NM, RD, PER>::run();
-        }
-    }
-};
-// ... and for the sub-step behind the barrier: LDS reads first, global->LDS loads in the MFMA slots after them
 template <int G, int NM, int RD, int PER, int NLD, int PER_V>
-struct SchedLast {
+struct SchedPhase {
     static __device__ __forceinline__ void run() {
         if constexpr (G < NM) {
             sched_group<SG_MFMA, 1>();
             constexpr int left = RD - G * PER;
-            constexpr int nds = left > PER ? PER : (left > 0 ? left : 0);
             constexpr int ds_slots = PER > 0 ? (RD + PER - 1) / PER : 0;
             constexpr int vleft = G >= ds_slots ? NLD - (G - ds_slots) * PER_V : 0;
-            sched_group<SG_DS_R, nds>();
+            sched_group<SG_DS_R, (left > PER ? PER : (left > 0 ? left : 0))>();
             sched_group<SG_VMEM_R, (vleft > PER_V ? PER_V : (vleft > 0 ? vleft : 0))>();
-            SchedLast<G + 1, NM, RD, PER, NLD, PER_V>::run();
+            SchedPhase<G + 1, NM, RD, PER, NLD, PER_V>::run();
         }
     }
 };
 
-template <bool A_KC, bool B_KC, typename OutT, int WAVES_M, int WAVES_N>
-__global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_d2l_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
-                                                                          OutT* __restrict__ C, int M, int N, int K, int64_t lda,
-                                                                          int64_t ldb, int64_t ldc, int accumulate, int tiles_m,
-                                                                          int tiles_n) {
-    constexpr int NW = WAVES_M * WAVES_N;
-    constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
-    constexpr int NKS = BK / 16;
+template <typename OutT> struct Out4;
+template <> struct Out4<bf16_t> { typedef bf16x4 type; };
+template <> struct Out4<float> { typedef f32x4 type; };
+
+// 8 waves (2 x 4), each owning 128 x 64 of the 256 x 256 block tile as 8 x 4 MFMA 16x16x32 tiles.  The 16x16x32 shape is
+// used because it sustains a higher clock than 32x32x16 under the board's power limit (fewer accumulator-register
+// accesses per flop).  A 64-wide K tile is worked off in four phases (k half, M half): a phase issues 16 MFMAs on 4 A and
+// 4 B fragments while the fragments of the next phase are read from LDS into the other register set.
+template <bool A_KC, bool B_KC, typename OutT>
+__global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B, OutT* __restrict__ C,
+                                                       int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
+                                                       int tiles_m, int tiles_n) {
+    constexpr int NW = 8, WAVES_N = 4;
     __shared__ __attribute__((aligned(1024))) bf16_t smem[4 * DTILE];  // A0 B0 A1 B1
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -361,34 +358,36 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_d2l_kernel(const 
     la.init(lane, wave, m0, M, lda);
     lb.init(lane, wave, n0, N, ldb);
 
-    f32x16 acc[TM][TN];
+    f32x4 acc[8][4];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
     const int nk = K / BK;
     const int64_t astep = A_KC ? BK : (int64_t)BK * lda;
     const int64_t bstep = B_KC ? BK : (int64_t)BK * ldb;
-    const int arow = wm * (TM * 32), brow = wn * (TN * 32);
+    const int arow = wm * 128, brow = wn * 64;
 
-    // Fragment reads go B first, then A: the first MFMAs of a sub-step need both B fragments and A[0] only, and LDS returns
-    // data in issue order, so the waits in front of those MFMAs cover the oldest reads instead of all of them.
-    bf16x8 fa[2][TM], fb[2][TN];
-    auto read_frags = [&](const bf16_t* sA, int ks, int buf) {
+    bf16x8 fa[2][4], fb[2][4];
+    auto read_a = [&](const bf16_t* sA, int ks, int half, int buf) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fb[buf][j] = sfrag<B_KC>(sA + DTILE, brow + j * 32, ks, lane);
-#pragma unroll
-        for (int i = 0; i < TM; ++i) fa[buf][i] = sfrag<A_KC>(sA, arow + i * 32, ks, lane);
+        for (int i = 0; i < 4; ++i) fa[buf][i] = sfrag<A_KC>(sA, arow + half * 64 + i * 16, ks, lane);
     };
-    auto mfmas = [&](int buf) {
+    auto read_b = [&](const bf16_t* sA, int ks, int buf) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int j = 0; j < 4; ++j) fb[buf][j] = sfrag<B_KC>(sA + DTILE, brow + j * 16, ks, lane);
+    };
+    // B is the first MFMA operand: the accumulator then holds C^T fragments, i.e. a lane owns 4 consecutive columns of one
+    // row of C, which it can store as one vector.
+    auto mfmas = [&](int half, int abuf, int bbuf) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[half * 4 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[bbuf][j], fa[abuf][i], acc[half * 4 + i][j], 0, 0, 0);
     };
     auto issue_tile = [&](int t, int stage) {
         la.issue(A + (int64_t)t * astep, smem + stage * 2 * DTILE, wave);
@@ -402,38 +401,39 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_d2l_kernel(const 
     asm volatile("" ::"s"(C), "s"(ldc), "s"(accumulate));
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
     __syncthreads();
-    read_frags(smem, 0, 0);
+    read_b(smem, 0, 0);
+    read_a(smem, 0, 0, 0);
 
-    constexpr int RD = (A_KC ? TM : 2 * TM) + (B_KC ? TN : 2 * TN);  // LDS reads per sub-step
-    constexpr int NM = TM * TN;                                      // MFMAs per sub-step
-    constexpr int NLD = 2 * (32 / NW);                               // global->LDS loads per wave and tile pair
-    // inner sub-steps: the reads of the next sub-step are issued behind the first MFMAs, leaving the last two MFMAs as slack
-#ifndef EZL_PER_MIN
-#define EZL_PER_MIN 1
-#endif
-    constexpr int PER0 = (RD + NM - 3) / (NM - 2);
-    constexpr int PER = PER0 > EZL_PER_MIN ? PER0 : EZL_PER_MIN;
-    // last sub-step: reads of the next tile's first fragments first, then the loads of tile kt+2
-    constexpr int PER_L = (RD + NM / 2 - 1) / (NM / 2);
-    constexpr int DS_SLOTS_L = (RD + PER_L - 1) / PER_L;
-    constexpr int PER_V = (NLD + (NM - DS_SLOTS_L) - 1) / (NM - DS_SLOTS_L);
+    constexpr int RA = A_KC ? 4 : 8, RB = B_KC ? 4 : 8;  // LDS reads per fragment set
+    constexpr int NM = 16;                                // MFMAs per phase
+    constexpr int NLD = 2 * (32 / NW);                    // global->LDS loads per wave and tile pair
+    // phases 0 and 2 fetch the A fragments of the other M half; phases 1 and 3 fetch B and A of the next k half
+#define EZL_PHASE_SCHED(RD, LD) SchedPhase<0, NM, (RD), ((RD) + 11) / 12, (LD), 2>::run()
 #define EZL_STEP(HAS_NEXT, DO_LOAD)                                                                       \
     {                                                                                                     \
         const int cur = kt & 1;                                                                           \
         const bf16_t* sA = smem + cur * 2 * DTILE;                                                         \
-        _Pragma("unroll") for (int ks = 0; ks < NKS - 1; ++ks) {                                          \
-            read_frags(sA, ks + 1, (ks + 1) & 1);                                                         \
-            mfmas(ks & 1);                                                                                \
-            SchedInner<0, NM, RD, PER>::run();                                                            \
-        }                                                                                                 \
+        read_a(sA, 0, 1, 1);                                                                              \
+        mfmas(0, 0, 0);                                                                                   \
+        EZL_PHASE_SCHED(RA, 0);                                                                           \
+        read_b(sA, 1, 1);                                                                                 \
+        read_a(sA, 1, 0, 0);                                                                              \
+        mfmas(1, 1, 0);                                                                                   \
+        EZL_PHASE_SCHED(RA + RB, 0);                                                                      \
+        read_a(sA, 1, 1, 1);                                                                              \
+        mfmas(0, 0, 1);                                                                                   \
+        EZL_PHASE_SCHED(RA, 0);                                                                           \
         __builtin_amdgcn_sched_barrier(0);                                                                \
         __builtin_amdgcn_s_waitcnt(0x0F70);                                                               \
         __syncthreads();                                                                                  \
         __builtin_amdgcn_sched_barrier(0);                                                                \
-        if (HAS_NEXT) read_frags(smem + (cur ^ 1) * 2 * DTILE, 0, 0);                                      \
+        if (HAS_NEXT) {                                                                                   \
+            read_b(smem + (cur ^ 1) * 2 * DTILE, 0, 0);                                                    \
+            read_a(smem + (cur ^ 1) * 2 * DTILE, 0, 0, 0);                                                 \
+        }                                                                                                 \
         if (DO_LOAD) issue_tile(kt + 2, cur);                                                             \
-        mfmas((NKS - 1) & 1);                                                                             \
-        SchedLast<0, NM, (HAS_NEXT) ? RD : 0, PER_L, (DO_LOAD) ? NLD : 0, PER_V>::run();                  \
+        mfmas(1, 1, 1);                                                                                   \
+        EZL_PHASE_SCHED((HAS_NEXT) ? RA + RB : 0, (DO_LOAD) ? NLD : 0);                                   \
         __builtin_amdgcn_sched_barrier(0);                                                                \
     }
 
@@ -445,16 +445,34 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_d2l_kernel(const 
     }
     EZL_STEP(false, false)
 #undef EZL_STEP
+#undef EZL_PHASE_SCHED
 
+    // epilogue: acc[i][j] register r is C[m0 + arow + 16 i + (lane & 15)][n0 + brow + 16 j + 4 (lane >> 4) + r]
+    typedef typename Out4<OutT>::type out4_t;
+    const bool vec_ok = (N % 4 == 0) && (ldc % 4 == 0) && (((uintptr_t)C & 15) == 0);
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < 8; ++i) {
+        const int row = m0 + arow + i * 16 + (lane & 15);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+        for (int j = 0; j < 4; ++j) {
+            const int col = n0 + brow + j * 16 + 4 * (lane >> 4);
+            if (row >= M || col >= N) continue;
+            OutT* dst = C + (int64_t)row * ldc + col;
+            if (vec_ok) {
+                out4_t v;
+                if (accumulate) {
+                    const out4_t old = *reinterpret_cast<const out4_t*>(dst);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm * (TM * 32) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (row < M && col < N) store_out<OutT>(C + (int64_t)row * ldc + col, acc[i][j][r], accumulate != 0);
+                    for (int r = 0; r < 4; ++r) v[r] = (OutT)(acc[i][j][r] + (float)old[r]);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] = (OutT)acc[i][j][r];
+                }
+                *reinterpret_cast<out4_t*>(dst) = v;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (col + r < N) store_out<OutT>(dst + r, acc[i][j][r], accumulate != 0);
             }
         }
     }
@@ -467,7 +485,7 @@ void launch(const void* A, const void* B, void* C, int M, int N, int K, int64_t 
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const dim3 grid((unsigned)(tiles_m * tiles_n)), block(512);
     if (K % BK == 0)
-        hipLaunchKernelGGL((gemm_d2l_kernel<A_KC, B_KC, OutT, 2, 4>), grid, block, 0, st, (const bf16_t*)A, (const bf16_t*)B,
+        hipLaunchKernelGGL((gemm_d2l_kernel<A_KC, B_KC, OutT>), grid, block, 0, st, (const bf16_t*)A, (const bf16_t*)B,
                            (OutT*)C, M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n);
     else
         hipLaunchKernelGGL((gemm_staged_kernel<A_KC, B_KC, OutT, true, 2, 4>), grid, block, 0, st, (const bf16_t*)A,

@@ -279,15 +279,51 @@ class EmbeddingFunction(torch.autograd.Function):
         return None, K.cast_f32_to_bf16(buf)
 
 
+def _raise_for_id_flag(bad, ids, num_embeddings):
+    if bad & 1:
+        raise ValueError("There is an input id in the input that is greater than the highest possible input id.\n"
+                         "Input: {}\nnum_embeddings: {}".format(ids, num_embeddings))
+    if bad & 2:
+        raise IndexError("negative token id in the input")
+
+
+# "sync": the check blocks on the gather, like the reference's host-side comparison (:107-109).
+# "deferred": the flag is copied to pinned host memory behind the gather and examined at the next
+# embedding call or flush_input_checks(); the launch queue never drains, the error surfaces one call late.
+_INPUT_CHECK = "sync"
+_PENDING_CHECKS = []
+
+
+def set_input_check(mode):
+    assert mode in ("sync", "deferred"), mode
+    global _INPUT_CHECK
+    flush_input_checks()
+    _INPUT_CHECK = mode
+
+
+def flush_input_checks(wait=True):
+    """Raise for any earlier embedding call whose out-of-range flag has arrived (all of them with wait=True)."""
+    while _PENDING_CHECKS:
+        ev, host, ids, n = _PENDING_CHECKS[0]
+        if not wait and not ev.query():
+            return
+        ev.synchronize()
+        _PENDING_CHECKS.pop(0)
+        _raise_for_id_flag(int(host.item()), ids, n)
+
+
 def embedding(ids, weight):
     """Row gather; raises ValueError for an id >= vocab like the reference (:107-109)."""
     out, flag = EmbeddingFunction.apply(ids, weight)
-    bad = int(flag.item())
-    if bad & 1:
-        raise ValueError("There is an input id in the input that is greater than the highest possible input id.\n"
-                         "Input: {}\nnum_embeddings: {}".format(ids, weight.shape[0]))
-    if bad & 2:
-        raise IndexError("negative token id in the input")
+    if _INPUT_CHECK == "deferred":
+        flush_input_checks(wait=False)
+        host = torch.empty(1, dtype=torch.int32, pin_memory=True)
+        host.copy_(flag, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        _PENDING_CHECKS.append((ev, host, ids, weight.shape[0]))
+        return out
+    _raise_for_id_flag(int(flag.item()), ids, weight.shape[0])
     return out
 
 

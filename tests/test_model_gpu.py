@@ -162,6 +162,19 @@ def test_bad_token_id_raises_value_error(gpu_device):
         emb(ids)
     out = emb(torch.tensor([[1, 2, 99]], device=gpu_device))
     assert torch.equal(out[0, 2], emb.weight[99])  # gather is bit-exact
+    # deferred mode: same error, raised when the flag is examined instead of inside the call
+    from easyllm_amd import functional
+    functional.set_input_check("deferred")
+    try:
+        emb(torch.tensor([[1, 2, 99]], device=gpu_device))
+        functional.flush_input_checks()
+        emb(ids)
+        with pytest.raises(ValueError):
+            functional.flush_input_checks()
+        functional.flush_input_checks()  # nothing left pending
+    finally:
+        functional._PENDING_CHECKS.clear()
+        functional.set_input_check("sync")
 
 
 def test_qkv_pack_and_bias_variants(gpu_device):
