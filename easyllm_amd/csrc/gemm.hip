@@ -408,7 +408,7 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
     constexpr int NM = 16;                                // MFMAs per phase
     constexpr int NLD = 2 * (32 / NW);                    // global->LDS loads per wave and tile pair
     // phases 0 and 2 fetch the A fragments of the other M half; phases 1 and 3 fetch B and A of the next k half
-#define EZL_PHASE_SCHED(RD, LD) SchedPhase<0, NM, (RD), ((RD) + 11) / 12, (LD), 2>::run()
+#define EZL_PHASE_SCHED(RD, LD) SchedPhase<0, NM, (RD), ((RD) + 11) / 12, (LD), 1>::run()
 #define EZL_STEP(HAS_NEXT, DO_LOAD)                                                                       \
     {                                                                                                     \
         const int cur = kt & 1;                                                                           \
