@@ -7,17 +7,16 @@
 //   dgrad     dX[T,in]  = dY[T,out] * W[out,in]      A k-contiguous, B n-contiguous
 //   wgrad     dW[out,in]= dY[T,out]^T * X[T,in]      A m-contiguous, B n-contiguous   (fp32 or bf16 out)
 //
-// Tiling: 256x256 block tile, K step 64, 8 waves (2x4), each wave owns 128x64 = 4x2 MFMA 32x32x16
-// tiles.  Operand tiles are double buffered in LDS (2 stages x 2 operands x 32 KiB).  An operand whose
-// reduction dimension is the strided one is kept as it lies in memory ([k][256]) and read with
-// ds_read_b64_tr_b16 (the LDS transpose read), so nothing is ever transposed in HBM.
+// Tiling: 256x256 block tile, K step 64, 8 waves (2x4), each wave owns 128x64.  Operand tiles are double buffered in LDS
+// (2 stages x 2 operands x 32 KiB).  An operand whose reduction dimension is the strided one is kept as it lies in
+// memory ([k][256]) and read with ds_read_b64_tr_b16 (the LDS transpose read), so nothing is ever transposed in HBM.
 //
-// Main kernel (K % 64 == 0): tiles go HBM -> LDS directly (global_load_lds_dwordx4, no staging
-// registers, no ds_write); bank conflicts are avoided by an XOR swizzle applied on the global-address
-// side.  The K loop is rotated: the barrier that publishes the next stage sits between the fragment
-// reads and the MFMAs of the last 16-wide sub-step, so the loads of tile kt+2 and the first fragment
-// reads of tile kt+1 are issued under those MFMAs; scheduler group barriers interleave one LDS read
-// per two MFMAs.  A second kernel with register staging and padded tiles covers K tails (K % 64 != 0).
+// Main kernel (K % 64 == 0): MFMA 16x16x32 (8x4 tiles per wave); tiles go HBM -> LDS directly
+// (global_load_lds_dwordx4, no staging registers, no ds_write); bank conflicts are avoided by an XOR swizzle applied on
+// the global-address side.  A K tile is consumed in four phases (k half x M half) of 16 MFMAs; the fragments of the
+// next phase are read during the current one, the barrier that publishes the next stage sits in front of the last
+// phase, and the loads of tile kt+2 are issued under that phase's MFMAs.  A second kernel with register staging,
+// padded tiles and MFMA 32x32x16 covers K tails (K % 64 != 0).
 // Blocks are renumbered so that each XCD (own L2) works on a contiguous band of tiles, 8 tiles tall.
 #include "common.h"
 
