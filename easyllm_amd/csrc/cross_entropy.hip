@@ -175,6 +175,98 @@ __global__ __launch_bounds__(kCeBlock) void ce_fused_kernel(const T* __restrict_
     }
 }
 
+// Fused loss + gradient for bf16 rows of up to 512 * 8 * NCH columns, held in registers: the kernel is bound by vector
+// ALU work as much as by HBM (a transcendental costs four issue slots), so exp(x - max) is computed once per element with
+// the bare v_exp_f32 (its argument is never positive; anything below 2^-126 may flush to zero) and kept in fp32 registers
+// for the gradient, vectors past the row end are filled with -inf instead of being branched around, and the raw
+// vectors of the block's next row are fetched while the current row is worked on.  HAS_CUT: columns [vend, V) are
+// excluded from max and sum but still receive their softmax gradient (reference semantics of cut_size).
+template <int NCH, bool HAS_CUT>
+__global__ __launch_bounds__(kCeBlock) void ce_fused_reg_kernel(const bf16_t* __restrict__ logits, const int64_t* __restrict__ labels,
+                                                                const float* __restrict__ weights, const float* __restrict__ count,
+                                                                float* __restrict__ loss, bf16_t* __restrict__ grad, int64_t rows,
+                                                                int V, int vend) {
+    __shared__ float red[kCeWaves];
+    const int v8 = V >> 3;
+    const float inv_n = 1.0f / count[0];
+    bf16x8 nxt[NCH];
+    auto fetch = [&](int64_t r) {
+        const bf16_t* src = logits + r * V;
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            const int i = threadIdx.x + j * kCeBlock;
+            if (i < v8) {
+                nxt[j] = ld_bf16x8(src + i * 8);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) nxt[j][k] = (bf16_t)(-INFINITY);
+            }
+        }
+    };
+    int64_t r = blockIdx.x;
+    if (r < rows) fetch(r);
+    for (; r < rows; r += gridDim.x) {
+        const float w = weights[r];
+        bf16_t* grow = grad + r * V;
+        const int64_t t = labels[r];
+        const bool masked = t < 0 || t >= vend;
+        const int tvec = masked ? -1 : (int)(t >> 3), tsub = (int)(t & 7);
+        float e[NCH][8];
+        float m = -INFINITY, xt = 0.f;
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            const int i = threadIdx.x + j * kCeBlock;
+            unpack8(nxt[j], e[j]);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                if (!HAS_CUT || i * 8 + k < vend) m = fmaxf(m, e[j][k]);
+            }
+            if (i == tvec) {  // exactly one thread holds the target logit
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    if (tsub == k) xt = e[j][k];
+            }
+        }
+        if (r + gridDim.x < rows) fetch(r + gridDim.x);
+        if (w == 0.f) {  // ignored position: exact zero gradient, contributes nothing to the loss
+            row_write_zero<bf16_t>(grow, V);
+            if (threadIdx.x == 0) loss[r] = 0.f;
+            continue;
+        }
+        m = block_max(m, red);
+        const float mb = m * kLog2e;
+        float ssum = 0.f;
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            const int i = threadIdx.x + j * kCeBlock;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                e[j][k] = __builtin_amdgcn_exp2f(e[j][k] * kLog2e - mb);
+                if (!HAS_CUT || i * 8 + k < vend) ssum += e[j][k];
+            }
+        }
+        ssum = block_sum(ssum, red);
+        xt = block_sum(xt, red);  // every other thread contributes 0
+        const float lse = m + logf(ssum);
+        if (threadIdx.x == 0) loss[r] = masked ? logf(ssum) : (lse - xt);
+        const float scale = w * inv_n;
+        const float ps = scale / ssum;  // exp(x - lse) * scale = e * scale / sum
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            const int i = threadIdx.x + j * kCeBlock;
+            float g[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) g[k] = e[j][k] * ps;
+            if (i == tvec) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    if (tsub == k) g[k] -= scale;
+            }
+            if (i < v8) st_bf16x8(grow + i * 8, pack8(g));
+        }
+    }
+}
+
 // weights[i] = mask[i] * (labels[i] != ignore_index); count[0] = sum(weights) -- one block, fixed order
 __global__ __launch_bounds__(1024) void ce_prepare_kernel(const int64_t* __restrict__ labels, const void* __restrict__ mask,
                                                           int mask_dtype, int64_t ignore_index, float* __restrict__ weights,
@@ -304,12 +396,18 @@ extern "C" int ezl_ce_fused(const void* logits, const void* labels, const void* 
     const size_t row_bytes = (size_t)V * (dtype == 0 ? 2 : 4);
     const bool in_lds = row_bytes <= 65536;
     hipStream_t st = (hipStream_t)stream;
-#define LAUNCH(TT, L)                                                                                                    \
-    hipLaunchKernelGGL((ce_fused_kernel<TT, L>), dim3(ce_grid(rows)), dim3(kCeBlock), (L) ? row_bytes : 0, st, (const TT*)logits, \
-                       (const int64_t*)labels, (const float*)weights, (const float*)count, (float*)loss_rows, (TT*)grad, rows, \
-                       V, vend)
-    if (dtype == 0) { if (in_lds) LAUNCH(bf16_t, true); else LAUNCH(bf16_t, false); }
-    else { if (in_lds) LAUNCH(float, true); else LAUNCH(float, false); }
+#define LAUNCH(KERNEL, TT, SMEM)                                                                                         \
+    hipLaunchKernelGGL((KERNEL), dim3(ce_grid(rows)), dim3(kCeBlock), SMEM, st, (const TT*)logits, (const int64_t*)labels, \
+                       (const float*)weights, (const float*)count, (float*)loss_rows, (TT*)grad, rows, V, vend)
+    if (dtype == 0) {
+        const bool cut = vend != V;
+        if (V <= kCeBlock * 8 * 2) { if (cut) LAUNCH((ce_fused_reg_kernel<2, true>), bf16_t, 0); else LAUNCH((ce_fused_reg_kernel<2, false>), bf16_t, 0); }
+        else if (V <= kCeBlock * 8 * 4) { if (cut) LAUNCH((ce_fused_reg_kernel<4, true>), bf16_t, 0); else LAUNCH((ce_fused_reg_kernel<4, false>), bf16_t, 0); }
+        else if (V <= kCeBlock * 8 * 8) { if (cut) LAUNCH((ce_fused_reg_kernel<8, true>), bf16_t, 0); else LAUNCH((ce_fused_reg_kernel<8, false>), bf16_t, 0); }
+        else LAUNCH((ce_fused_kernel<bf16_t, false>), bf16_t, 0);
+    } else {
+        if (in_lds) LAUNCH((ce_fused_kernel<float, true>), float, row_bytes); else LAUNCH((ce_fused_kernel<float, false>), float, 0);
+    }
 #undef LAUNCH
     EZL_LAUNCH_CHECK("ezl_ce_fused");
     return EZL_OK;

@@ -14,7 +14,10 @@ inline unsigned grid_for(int64_t items, int per_block, int64_t cap = 256 * 32) {
     return (unsigned)g;
 }
 
-__device__ __forceinline__ float sigmoidf_fast(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// 1 / (1 + 2^(-x log2 e)) with the bare exp2 / rcp instructions (1 ulp each); saturates correctly at both ends
+__device__ __forceinline__ float sigmoidf_fast(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+}
 
 // ---------------------------------------------------------------------------------------------
 // SwiGLU: out = silu(gate) * up     (llama/transformer.py:220-222, glu_activations.py:56-61)
