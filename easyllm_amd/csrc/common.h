@@ -74,21 +74,35 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-// out[col] (+)= sum_r partial[r][col];  64 columns per block, 4 row groups folded through LDS.
+// out[col] (+)= sum_r partial[r][col];  64 columns per block, 16 row groups (loads of a group issued eight at a time)
+// folded through LDS in a fixed order.
+constexpr int kColsumThreads = 1024;
 template <int UNUSED>
-__global__ __launch_bounds__(256) void ezl_colsum_kernel(const float* __restrict__ partial, int nrows, int ncols,
-                                                     bf16_t* __restrict__ out_bf16, float* __restrict__ out_f32,
-                                                     int accumulate) {
-    __shared__ float s[4][64];
+__global__ __launch_bounds__(kColsumThreads) void ezl_colsum_kernel(const float* __restrict__ partial, int nrows, int ncols,
+                                                                    bf16_t* __restrict__ out_bf16, float* __restrict__ out_f32,
+                                                                    int accumulate) {
+    constexpr int G = kColsumThreads / 64;
+    __shared__ float s[G][64];
     const int c = threadIdx.x & 63, g = threadIdx.x >> 6;
     const int col = blockIdx.x * 64 + c;
     float acc = 0.f;
-    if (col < ncols)
-        for (int r = g; r < nrows; r += 4) acc += partial[(size_t)r * ncols + col];
+    if (col < ncols) {
+        int r = g;
+        for (; r + 7 * G < nrows; r += 8 * G) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = partial[(size_t)(r + u * G) * ncols + col];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += v[u];
+        }
+        for (; r < nrows; r += G) acc += partial[(size_t)r * ncols + col];
+    }
     s[g][c] = acc;
     __syncthreads();
     if (g == 0 && col < ncols) {
-        const float v = s[0][c] + s[1][c] + s[2][c] + s[3][c];
+        float v = 0.f;
+#pragma unroll
+        for (int i = 0; i < G; ++i) v += s[i][c];
         if (out_f32) out_f32[col] = accumulate ? out_f32[col] + v : v;
         else out_bf16[col] = (bf16_t)v;
     }

@@ -436,7 +436,7 @@ extern "C" int ezl_bias_grad(const void* dy, void* db_bf16, void* db_f32, int ac
     hipLaunchKernelGGL(bias_grad_partial_kernel, grid, dim3(kBlock), 0, (hipStream_t)stream, (const bf16_t*)dy, (float*)workspace,
                        rows, (int)n);
     EZL_LAUNCH_CHECK("ezl_bias_grad");
-    hipLaunchKernelGGL(ezl_colsum_kernel<0>, dim3((unsigned)((n + 63) / 64)), dim3(256), 0, (hipStream_t)stream,
+    hipLaunchKernelGGL(ezl_colsum_kernel<0>, dim3((unsigned)((n + 63) / 64)), dim3(kColsumThreads), 0, (hipStream_t)stream,
                        (const float*)workspace, 64, (int)n, (bf16_t*)db_bf16, (float*)db_f32, accumulate);
     EZL_LAUNCH_CHECK("ezl_bias_grad(colsum)");
     return EZL_OK;

@@ -105,19 +105,37 @@ __global__ __launch_bounds__(1024) void rmsnorm_bwd_kernel(const bf16_t* __restr
     }
     int parity = 0;
     const float inv_h = 1.0f / (float)h;
-    for (int row0 = blockIdx.x * rpb; row0 < T; row0 += gridDim.x * rpb) {
+    // The operands of the block's next rows are requested before the current rows are reduced, so HBM reads stay in
+    // flight across the barrier of the row reduction.
+    bf16x8 xr[NCHUNK], dyr[NCHUNK], drr[NCHUNK];
+    auto fetch = [&](int row0, bf16x8* xo, bf16x8* dyo, bf16x8* dro) {
+        const int row = row0 + slot;
+        const size_t base = (size_t)row * h;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            const int col = (c * tpr + tin) * 8;
+            if (row < T && col < h) {
+                xo[c] = ld_bf16x8(x + base + col);
+                dyo[c] = ld_bf16x8(dy + base + col);
+                if (HAS_DRES) dro[c] = ld_bf16x8(dres + base + col);
+            }
+        }
+    };
+    const int stride = gridDim.x * rpb;
+    int row0 = blockIdx.x * rpb;
+    if (row0 < T) fetch(row0, xr, dyr, drr);
+    for (; row0 < T; row0 += stride) {
         const int row = row0 + slot;
         const bool live = row < T;
         const size_t base = (size_t)row * h;
         const float rs = live ? rstd[row] : 0.f;
-        bf16x8 xr[NCHUNK], dyr[NCHUNK];
+        bf16x8 xn[NCHUNK], dyn[NCHUNK], drn[NCHUNK];
+        if (row0 + stride < T) fetch(row0 + stride, xn, dyn, drn);
         float dot = 0.f;
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
             const int col = (c * tpr + tin) * 8;
             if (live && col < h) {
-                xr[c] = ld_bf16x8(x + base + col);
-                dyr[c] = ld_bf16x8(dy + base + col);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) dot += (float)dyr[c][i] * wv[c][i] * ((float)xr[c][i] * rs);
             }
@@ -136,18 +154,22 @@ __global__ __launch_bounds__(1024) void rmsnorm_bwd_kernel(const bf16_t* __restr
             const int col = (c * tpr + tin) * 8;
             if (live && col < h) {
                 float o[8];
-                float dr[8];
-                if (HAS_DRES) unpack8(ld_bf16x8(dres + base + col), dr);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const float xhat = (float)xr[c][i] * rs;
                     const float dyv = (float)dyr[c][i];
                     o[i] = rs * (dyv * wv[c][i] - xhat * cmean);
-                    if (HAS_DRES) o[i] += dr[i];
+                    if (HAS_DRES) o[i] += (float)drr[c][i];
                     dwacc[c][i] += dyv * xhat;
                 }
                 st_bf16x8(dx + base + col, pack8(o));
             }
+        }
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            xr[c] = xn[c];
+            dyr[c] = dyn[c];
+            if (HAS_DRES) drr[c] = drn[c];
         }
     }
     // fold the row slots of this block: slot 0 stores, the others add, one barrier per slot
@@ -247,7 +269,7 @@ extern "C" int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight
     }
 #undef LAUNCH
     EZL_LAUNCH_CHECK("ezl_rmsnorm_bwd");
-    hipLaunchKernelGGL(ezl_colsum_kernel<0>, dim3((unsigned)((h + 63) / 64)), dim3(256), 0, st, (const float*)workspace,
+    hipLaunchKernelGGL(ezl_colsum_kernel<0>, dim3((unsigned)((h + 63) / 64)), dim3(kColsumThreads), 0, st, (const float*)workspace,
                        (int)grid, (int)h, (bf16_t*)dw_bf16, (float*)dw_f32, accumulate);
     EZL_LAUNCH_CHECK("ezl_rmsnorm_bwd(colsum)");
     return EZL_OK;
