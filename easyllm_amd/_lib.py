@@ -37,12 +37,16 @@ SIGNATURES = {
     "ezl_ce_fused": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
     "ezl_ce_reduce": [_vp, _vp, _vp, _vp, _i64, _vp],
     "ezl_scale_by_scalar": [_vp, _vp, _i64, _i32, _vp],
+    "ezl_sumsq_f32": [_vp, _i64, _vp, _vp],
+    "ezl_clip_coef": [_vp, _i64, _f32, _vp, _vp],
+    "ezl_adamw_step": [_vp, _vp, _vp, _vp, _vp, _i64, _f32, _f32, _f32, _f32, _f32, _i64, _i32, _vp, _vp],
 }
 _SPECIAL = {
     "ezl_version": ([], ctypes.c_int),
     "ezl_last_error": ([], ctypes.c_char_p),
     "ezl_rmsnorm_bwd_workspace_bytes": ([_i64, _i64], _i64),
     "ezl_bias_grad_workspace_bytes": ([_i64, _i64], _i64),
+    "ezl_sumsq_partials": ([], _i64),
 }
 
 _lib = None
@@ -88,3 +92,7 @@ def rmsnorm_bwd_workspace_bytes(rows, h):
 
 def bias_grad_workspace_bytes(rows, n):
     return load().ezl_bias_grad_workspace_bytes(rows, n)
+
+
+def sumsq_partials():
+    return load().ezl_sumsq_partials()

@@ -377,3 +377,45 @@ def scale_by_scalar_(x, scalar):
     _need(x.is_contiguous() and x.dtype in (BF16, torch.float32), "x must be contiguous bf16/fp32")
     _lib.call("ezl_scale_by_scalar", _p(x), _p(scalar), x.numel(), 0 if x.dtype == BF16 else 1, _stream())
     return x
+
+
+# ------------------------------------------------------------------------------------- optimizer step
+def _f32c(t, name):
+    _need(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous(), "%s must be a contiguous fp32 GPU tensor" % name)
+
+
+def sumsq_partials():
+    return int(_lib.sumsq_partials())
+
+
+def sumsq(x, partials_row):
+    """partials_row (fp32 [sumsq_partials()]) <- per-block sums of x^2."""
+    _f32c(x, "x"); _f32c(partials_row, "partials")
+    _need(partials_row.numel() == sumsq_partials(), "partials row has the wrong length")
+    _lib.call("ezl_sumsq_f32", _p(x), x.numel(), _p(partials_row), _stream())
+
+
+def clip_coef(partials, max_norm, out=None):
+    """-> fp32 [2] on the GPU: (global L2 norm, clip coefficient)."""
+    _f32c(partials, "partials")
+    if out is None:
+        out = torch.empty(2, dtype=torch.float32, device=partials.device)
+    _lib.call("ezl_clip_coef", _p(partials), partials.numel(), float(max_norm), _p(out), _stream())
+    return out
+
+
+def adamw_step(master, exp_avg, exp_avg_sq, grad, param, lr, beta1, beta2, eps, weight_decay, step, bias_correction=True,
+               norm_coef=None):
+    """In-place AdamW update of (master, exp_avg, exp_avg_sq) from fp32 grad; param (bf16 or None) is refreshed from master."""
+    for t, n in ((master, "master"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq"), (grad, "grad")):
+        _f32c(t, n)
+        _need(t.numel() == master.numel(), "%s size mismatch" % n)
+    if param is not None:
+        _bf16c(param, "param")
+        _need(param.numel() == master.numel(), "param size mismatch")
+    if norm_coef is not None:
+        _f32c(norm_coef, "norm_coef")
+        _need(norm_coef.numel() == 2, "norm_coef must hold (norm, coefficient)")
+    _lib.call("ezl_adamw_step", _p(master), _p(exp_avg), _p(exp_avg_sq), _p(grad), _p(param), master.numel(), float(lr),
+              float(beta1), float(beta2), float(eps), float(weight_decay), int(step), 1 if bias_correction else 0,
+              _p(norm_coef), _stream())

@@ -119,6 +119,21 @@ int ezl_ce_reduce(const void* loss_rows, const void* weights, const void* count,
 /* x *= scalar[0] unless scalar[0] == 1 (applies the upstream gradient of the fused loss) */
 int ezl_scale_by_scalar(void* x, const void* scalar_f32, int64_t n, int dtype, void* stream);
 
+/* ---- optimizer step: apex FusedAdam in AdamW mode under DeepSpeed's bf16 optimizer with gradient clipping
+ *      (llm/utils/model/optimizer_helper.py:70-98; configs/megatron/llama_7b_sft.yaml:13,106-112) ----
+ * sumsq:     partials[0 .. ezl_sumsq_partials()) = per-block sums of x[i]^2 (fp32 x, every slot written).
+ * clip_coef: norm_coef_out[0] = sqrt(sum of `count` partials) (fixed order), norm_coef_out[1] = max_norm / (norm + 1e-6)
+ *            if that is < 1, else 1 (max_norm <= 0: no clipping).
+ * adamw:     g = grad * norm_coef[1] (1 if norm_coef is NULL); m = b1 m + (1-b1) g; v = b2 v + (1-b2) g^2;
+ *            master -= lr * (m/bc1 / (sqrt(v/bc2) + eps) + weight_decay * master), bc = 1 - beta^step (1 without bias
+ *            correction); param_bf16 (may be NULL) = round-to-nearest-even of the new master value. */
+int64_t ezl_sumsq_partials(void);
+int ezl_sumsq_f32(const void* x, int64_t n, void* partials, void* stream);
+int ezl_clip_coef(const void* partials, int64_t count, float max_norm, void* norm_coef_out, void* stream);
+int ezl_adamw_step(void* master, void* exp_avg, void* exp_avg_sq, const void* grad, void* param_bf16, int64_t n, float lr,
+                   float beta1, float beta2, float eps, float weight_decay, int64_t step, int bias_correction,
+                   const void* norm_coef, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -21,6 +21,9 @@ against library routines, closed forms and invariants:
   cross entropy ........ pinned (``F.cross_entropy``, uniform-logits ln V, shift invariance)
   dynamic-ckpt rule .... pinned (table-driven known answers written from the reference text)
   packed inputs ........ pinned (hand-worked known answers)
+  optimizer step ....... pinned (``torch.optim.AdamW`` over several steps with and without weight decay,
+                                ``torch.nn.utils.clip_grad_norm_``); apex / DeepSpeed themselves are absent, so
+                                their rounding order inside the update is parity unpinned
 
 Parity unpinned (defined by code that is neither under /root/reference nor installed): DeepSpeed's
 micro-batch loss scaling / bf16-optimizer accumulation / checkpoint internals, and flash-attn 2.2.5's
@@ -382,6 +385,34 @@ def packed_doc_lengths(total, lo, hi, seed):
         lens.append(ln)
         acc += ln
     return lens
+
+
+# --------------------------------------------------------------------------------------------
+# optimizer step (apex FusedAdam in AdamW mode + DeepSpeed global-norm clipping;
+# llm/utils/model/optimizer_helper.py:70-98, configs/megatron/llama_7b_sft.yaml:13,106-112)
+# --------------------------------------------------------------------------------------------
+def global_grad_norm(grads):
+    """L2 norm over all gradient tensors."""
+    return math.sqrt(sum(float((g.double() ** 2).sum()) for g in grads))
+
+
+def clip_coefficient(total_norm, max_norm):
+    """DeepSpeed: clip_coef = max_norm / (total_norm + 1e-6), applied only when below one."""
+    if max_norm <= 0:
+        return 1.0
+    c = max_norm / (total_norm + 1e-6)
+    return c if c < 1.0 else 1.0
+
+
+def adamw_step(p, m, v, g, lr, beta1, beta2, eps, weight_decay, step, bias_correction=True):
+    """One AdamW update (decoupled weight decay); returns new (p, m, v).  step counts from 1."""
+    m = beta1 * m + (1.0 - beta1) * g
+    v = beta2 * v + (1.0 - beta2) * g * g
+    bc1 = 1.0 - beta1 ** step if bias_correction else 1.0
+    bc2 = 1.0 - beta2 ** step if bias_correction else 1.0
+    denom = (v / bc2).sqrt() + eps
+    p = p - lr * ((m / bc1) / denom + weight_decay * p)
+    return p, m, v
 
 
 # --------------------------------------------------------------------------------------------

@@ -189,3 +189,40 @@ def test_checkpoint_function_recomputes_and_matches(monkeypatch):
     lin.weight.grad = None
     chunk(x, aux)[0].sum().backward()
     assert torch.equal(g1, x.grad) and torch.equal(gw1, lin.weight.grad)
+
+
+def test_weight_decay_split_and_optimizer_config_errors():
+    """optimizer_helper.py:19-51,70-72: biases and MixedFusedLayerNorm modules get no decay (RMSNorm weights do, as in
+    the reference); cpu_optimizer is refused."""
+    import torch
+    from easyllm_amd import optimizer
+    from easyllm_amd.layers import RMSNorm
+
+    class MixedFusedLayerNorm(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.weight = torch.nn.Parameter(torch.ones(4))
+
+    class Toy(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = torch.nn.Linear(4, 4, bias=True)
+            self.norm = RMSNorm(True, 4)
+            self.ln = MixedFusedLayerNorm()
+            self.frozen = torch.nn.Linear(4, 4, bias=False)
+            self.frozen.weight.requires_grad = False
+
+    toy = Toy()
+    decay, no_decay = optimizer.get_params_for_weight_decay_optimization(toy)
+    assert {id(p) for p in decay["params"]} == {id(toy.lin.weight), id(toy.frozen.weight), id(toy.norm.weight)}
+    assert {id(p) for p in no_decay["params"]} == {id(toy.lin.bias), id(toy.ln.weight)} and no_decay["weight_decay"] == 0.0
+    groups = optimizer.filter_freeze_param_groups([{"params": [toy.frozen.weight]}, decay])
+    assert len(groups) == 1 and groups[0] is decay
+    with pytest.raises(NotImplementedError):
+        optimizer.build_optimizer({"type": "FusedAdam", "cpu_optimizer": True, "kwargs": {}}, toy)
+    with pytest.raises(NotImplementedError):
+        optimizer.build_optimizer({"type": "SophiaG", "kwargs": {}}, toy)
+    with pytest.raises(RuntimeError):
+        optimizer.FusedAdam([toy.lin.weight], amsgrad=True)
+    with pytest.raises(ValueError):  # parameters without fp32 gradient buffers are rejected before any GPU work
+        optimizer.FusedAdam([toy.lin.weight])

@@ -360,3 +360,40 @@ def test_step_flops_table():
     c1 = dict(num_layers=2, hidden_size=256, num_attention_heads=4, num_kv_attention_heads=4, head_dim=64,
               intermediate_size=688, vocab_size=32000)
     assert abs(O.step_flops(c1, 2, 512) / 6.166e10 - 1) < 1e-3
+
+
+# ------------------------------------------------------------------------------------- optimizer step
+@pytest.mark.parametrize("wd", [0.0, 0.1])
+def test_adamw_step_matches_torch_adamw(wd):
+    g = torch.Generator().manual_seed(21)
+    p0 = torch.randn(257, generator=g, dtype=torch.float64)
+    ref_p = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.AdamW([ref_p], lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=wd)
+    p, m, v = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    for step in range(1, 6):
+        grad = torch.randn(257, generator=g, dtype=torch.float64) * (0.1 if step % 2 else 3.0)
+        ref_p.grad = grad.clone()
+        opt.step()
+        p, m, v = O.adamw_step(p, m, v, grad, 3e-3, 0.9, 0.95, 1e-8, wd, step)
+        assert torch.allclose(p, ref_p.detach(), rtol=1e-12, atol=1e-14), step
+    # without bias correction the first update is lr * (1-b1) g / (sqrt((1-b2)) |g| + eps)
+    p1, _, _ = O.adamw_step(torch.zeros(3, dtype=torch.float64), torch.zeros(3, dtype=torch.float64),
+                            torch.zeros(3, dtype=torch.float64), torch.tensor([2.0, -4.0, 0.0], dtype=torch.float64),
+                            1.0, 0.9, 0.99, 0.0, 0.0, 1, bias_correction=False)
+    assert torch.allclose(p1[:2], torch.tensor([-1.0, 1.0], dtype=torch.float64))  # 0.1 g / (0.1 |g|)
+
+
+def test_global_norm_and_clip_match_torch():
+    g = torch.Generator().manual_seed(22)
+    grads = [torch.randn(50, 7, generator=g), torch.randn(13, generator=g) * 5, torch.zeros(4)]
+    params = [torch.nn.Parameter(torch.zeros_like(x)) for x in grads]
+    for p_, x in zip(params, grads):
+        p_.grad = x.clone()
+    total = torch.nn.utils.clip_grad_norm_(params, max_norm=1.0)
+    norm = O.global_grad_norm(grads)
+    assert abs(norm - float(total)) <= 1e-5 * norm
+    c = O.clip_coefficient(norm, 1.0)
+    for p_, x in zip(params, grads):
+        assert torch.allclose(p_.grad, x * c, rtol=1e-5, atol=1e-7)
+    assert O.clip_coefficient(0.5, 1.0) == 1.0 and O.clip_coefficient(3.0, 0.0) == 1.0
+    assert abs(O.clip_coefficient(4.0, 1.0) - 1.0 / (4.0 + 1e-6)) < 1e-15
