@@ -104,6 +104,11 @@ class FusedAdam:
                     p.data.copy_(st["master"])
         return norm_coef
 
+    def refresh_fp32_params(self):
+        """Re-reads the fp32 master copies from the model weights (called after a checkpoint was loaded into them)."""
+        for _, p in self._all_params():
+            self.state[p]["master"].copy_(p.detach().float())
+
     def zero_grad(self, set_to_none=True):
         """No memset: the next gradient written to each main_grad overwrites it."""
         for _, p in self._all_params():
