@@ -39,6 +39,7 @@ SIGNATURES = {
     "ezl_scale_by_scalar": [_vp, _vp, _i64, _i32, _vp],
     "ezl_sumsq_f32": [_vp, _i64, _vp, _vp],
     "ezl_clip_coef": [_vp, _i64, _f32, _vp, _vp],
+    "ezl_build_location_idx": [_vp, _i64, _vp, _i64, _i64, _i64, _i64, _vp, _i64],
     "ezl_adamw_step": [_vp, _vp, _vp, _vp, _vp, _i64, _f32, _f32, _f32, _f32, _f32, _i64, _i32, _vp, _vp],
 }
 _SPECIAL = {
@@ -47,6 +48,7 @@ _SPECIAL = {
     "ezl_rmsnorm_bwd_workspace_bytes": ([_i64, _i64], _i64),
     "ezl_bias_grad_workspace_bytes": ([_i64, _i64], _i64),
     "ezl_sumsq_partials": ([], _i64),
+    "ezl_location_idx_rows": ([_i64, _i64, _i64], _i64),
 }
 
 _lib = None
@@ -96,3 +98,7 @@ def bias_grad_workspace_bytes(rows, n):
 
 def sumsq_partials():
     return load().ezl_sumsq_partials()
+
+
+def location_idx_rows(seq_length, num_epochs, tokens_per_epoch):
+    return load().ezl_location_idx_rows(seq_length, num_epochs, tokens_per_epoch)

@@ -134,6 +134,15 @@ int ezl_adamw_step(void* master, void* exp_avg, void* exp_avg_sq, const void* gr
                    float beta1, float beta2, float eps, float weight_decay, int64_t step, int bias_correction,
                    const void* norm_coef, void* stream);
 
+/* ---- packed-sequence sample index (host code, no GPU): llm/data/cores/helpers.cpp:36-122 `build_location_idx`
+ *      (python twin llm/data/nlp_dataset.py:424-463) ----
+ * rows:  (num_epochs * tokens_per_epoch - 1) / seq_length + 1, or -1 for arguments the reference asserts against.
+ * build: out[k] = (position in doc_idx, token offset in that document) of the first token of sample k, samples being
+ *        seq_length + 1 tokens long and overlapping by one token; int32 [rows][2].  All indices are bounds-checked. */
+int64_t ezl_location_idx_rows(int64_t seq_length, int64_t num_epochs, int64_t tokens_per_epoch);
+int ezl_build_location_idx(const int32_t* sizes, int64_t n_sizes, const int32_t* doc_idx, int64_t n_doc_idx, int64_t seq_length,
+                           int64_t num_epochs, int64_t tokens_per_epoch, int32_t* out, int64_t out_rows);
+
 #ifdef __cplusplus
 }
 #endif

@@ -21,6 +21,8 @@ against library routines, closed forms and invariants:
   cross entropy ........ pinned (``F.cross_entropy``, uniform-logits ln V, shift invariance)
   dynamic-ckpt rule .... pinned (table-driven known answers written from the reference text)
   packed inputs ........ pinned (hand-worked known answers)
+  sample locations ..... pinned (the reference's own helpers.cpp compiled into oracle/_ref by oracle/build_ref.py, and
+                                slicing the concatenated token stream by brute force)
   optimizer step ....... pinned (``torch.optim.AdamW`` over several steps with and without weight decay,
                                 ``torch.nn.utils.clip_grad_norm_``); apex / DeepSpeed themselves are absent, so
                                 their rounding order inside the update is parity unpinned
@@ -385,6 +387,21 @@ def packed_doc_lengths(total, lo, hi, seed):
         lens.append(ln)
         acc += ln
     return lens
+
+
+# --------------------------------------------------------------------------------------------
+# packed-sequence sample locations (llm/data/cores/helpers.cpp:36-122, nlp_dataset.py:424-463)
+# --------------------------------------------------------------------------------------------
+def build_location_idx(sizes, doc_idx, seq_length, num_epochs, tokens_per_epoch):
+    """Closed form: samples of seq_length + 1 tokens overlap by one token, so sample k starts at token k * seq_length
+    of the documents laid end to end in doc_idx order; row k = (position in doc_idx, offset inside that document)."""
+    sizes, doc_idx = np.asarray(sizes, dtype=np.int64), np.asarray(doc_idx, dtype=np.int64)
+    num_samples = (num_epochs * tokens_per_epoch - 1) // seq_length
+    ends = np.cumsum(sizes[doc_idx])                                  # one past each document's last token
+    starts = np.arange(num_samples + 1, dtype=np.int64) * seq_length
+    where = np.searchsorted(ends, starts, side="right")               # first document whose end lies beyond the token
+    before = np.concatenate(([0], ends))[where]
+    return np.stack([where, starts - before], axis=1).astype(np.int32)
 
 
 # --------------------------------------------------------------------------------------------
