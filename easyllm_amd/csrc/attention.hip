@@ -624,7 +624,7 @@ int check_common(const char* name, int64_t T, int64_t s_len, int64_t nq, int64_t
                  int nstrides) {
     EZL_REQUIRE(d == 64 || d == 128, EZL_EUNSUPPORTED, "%s: head dim must be 64 or 128 (got %lld)", name, (long long)d);
     EZL_REQUIRE(nq > 0 && nk > 0 && nq % nk == 0, EZL_EINVAL, "%s: nq must be a positive multiple of nk", name);
-    EZL_REQUIRE(T >= 0 && T < (1LL << 30) && s_len > 0 && T % s_len == 0 && ndocs > 0 && ndocs < (1LL << 24), EZL_EINVAL,
+    EZL_REQUIRE(T >= 0 && T < (1LL << 30) && (T == 0 || (s_len > 0 && T % s_len == 0)) && ndocs > 0 && ndocs < (1LL << 24), EZL_EINVAL,
                 "%s: bad token / document counts", name);
     EZL_REQUIRE(nq < 65536, EZL_EUNSUPPORTED, "%s: too many heads", name);
     for (int i = 0; i < nstrides; ++i) EZL_REQUIRE(strides[i] % 8 == 0, EZL_EINVAL, "%s: strides must be multiples of 8 elements", name);

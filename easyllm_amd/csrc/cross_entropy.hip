@@ -338,7 +338,7 @@ inline unsigned ce_grid(int64_t rows) { return (unsigned)(rows < 256 * 8 ? (rows
 
 extern "C" int ezl_ce_prepare(const void* labels, const void* loss_mask, int mask_dtype, int64_t ignore_index, void* weights,
                               void* count, int64_t n, void* stream) {
-    EZL_REQUIRE(n >= 0 && labels && weights && count, EZL_EINVAL, "ezl_ce_prepare: null pointer");
+    EZL_REQUIRE(n >= 0 && count && (n == 0 || (labels && weights)), EZL_EINVAL, "ezl_ce_prepare: null pointer");
     EZL_REQUIRE(mask_dtype >= 0 && mask_dtype <= 4 && (mask_dtype == 0 || loss_mask), EZL_EINVAL, "ezl_ce_prepare: bad loss_mask");
     hipLaunchKernelGGL(ce_prepare_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const int64_t*)labels, loss_mask,
                        mask_dtype, ignore_index, (float*)weights, (float*)count, n);
@@ -415,7 +415,7 @@ extern "C" int ezl_ce_fused(const void* logits, const void* labels, const void* 
 
 extern "C" int ezl_ce_reduce(const void* loss_rows, const void* weights, const void* count, void* loss_out, int64_t n,
                              void* stream) {
-    EZL_REQUIRE(n >= 0 && loss_rows && weights && count && loss_out, EZL_EINVAL, "ezl_ce_reduce: null pointer");
+    EZL_REQUIRE(n >= 0 && count && loss_out && (n == 0 || (loss_rows && weights)), EZL_EINVAL, "ezl_ce_reduce: null pointer");
     hipLaunchKernelGGL(ce_reduce_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const float*)loss_rows,
                        (const float*)weights, (const float*)count, (float*)loss_out, n);
     EZL_LAUNCH_CHECK("ezl_ce_reduce");

@@ -317,8 +317,8 @@ extern "C" int ezl_rope_apply(const void* x, void* out, const void* cos_table, c
     EZL_REQUIRE(in_row_stride % 8 == 0 && out_row_stride % 8 == 0 && in_row_stride >= nheads * d && out_row_stride >= nheads * d,
                 EZL_EINVAL, "ezl_rope_apply: bad row stride");
     EZL_REQUIRE(npos >= 1 && (position_ids || npos >= s), EZL_EINVAL, "ezl_rope_apply: cos/sin table shorter than the sequence");
-    EZL_REQUIRE(x && out && cos_table && sin_table && ezl_aligned16(x) && ezl_aligned16(out) && ezl_aligned16(cos_table) &&
-                    ezl_aligned16(sin_table),
+    EZL_REQUIRE((s == 0 || (x && out)) && cos_table && sin_table && ezl_aligned16(x) && ezl_aligned16(out) &&
+                    ezl_aligned16(cos_table) && ezl_aligned16(sin_table),
                 EZL_EINVAL, "ezl_rope_apply: null or misaligned pointer");
     EZL_REQUIRE(s < (1LL << 31) && b < (1LL << 31), EZL_EUNSUPPORTED, "ezl_rope_apply: shape too large");
     if (s == 0) return EZL_OK;

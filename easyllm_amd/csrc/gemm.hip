@@ -491,6 +491,13 @@ void launch(const void* A, const void* B, void* C, int M, int N, int K, int64_t 
                            (const bf16_t*)B, (OutT*)C, M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n);
 }
 
+// C = 0 for an empty reduction (a fill kernel rather than a memset node, so the call can be captured into a graph)
+template <typename OutT>
+__global__ __launch_bounds__(256) void zero_c_kernel(OutT* __restrict__ C, int64_t M, int64_t N, int64_t ldc) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < M * N; i += (int64_t)gridDim.x * 256)
+        C[(i / N) * ldc + (i % N)] = (OutT)0.0f;
+}
+
 }  // namespace
 
 
@@ -502,8 +509,17 @@ extern "C" int ezl_gemm_bf16(const void* A, const void* B, void* C, int64_t M, i
     EZL_REQUIRE(M >= 0 && N >= 0 && K >= 0, EZL_EINVAL, "ezl_gemm_bf16: negative size");
     EZL_REQUIRE(out_dtype == 0 || out_dtype == 1, EZL_EUNSUPPORTED, "ezl_gemm_bf16: out_dtype must be 0 (bf16) or 1 (fp32)");
     if (M == 0 || N == 0) return EZL_OK;
-    EZL_REQUIRE(K > 0, EZL_EUNSUPPORTED, "ezl_gemm_bf16: K must be positive");
-    EZL_REQUIRE(A && B && C, EZL_EINVAL, "ezl_gemm_bf16: null pointer");
+    EZL_REQUIRE(C, EZL_EINVAL, "ezl_gemm_bf16: null pointer");
+    if (K == 0) {  // empty reduction (a weight gradient over zero tokens): C = 0, or C unchanged when accumulating
+        EZL_REQUIRE(ldc >= N, EZL_EINVAL, "ezl_gemm_bf16: leading dimension too small");
+        if (!accumulate) {
+            if (out_dtype == 0) hipLaunchKernelGGL(zero_c_kernel<bf16_t>, dim3(256), dim3(256), 0, (hipStream_t)stream, (bf16_t*)C, M, N, ldc);
+            else hipLaunchKernelGGL(zero_c_kernel<float>, dim3(256), dim3(256), 0, (hipStream_t)stream, (float*)C, M, N, ldc);
+            EZL_LAUNCH_CHECK("ezl_gemm_bf16(zero)");
+        }
+        return EZL_OK;
+    }
+    EZL_REQUIRE(A && B, EZL_EINVAL, "ezl_gemm_bf16: null pointer");
     EZL_REQUIRE(ezl_aligned16(A) && ezl_aligned16(B) && lda % 8 == 0 && ldb % 8 == 0, EZL_EINVAL,
                 "ezl_gemm_bf16: operands must be 16-byte aligned with leading dimensions that are multiples of 8");
     // every 128-bit chunk must lie wholly inside or wholly outside the matrix

@@ -203,7 +203,7 @@ extern "C" int ezl_rmsnorm_fwd(const void* x, const void* residual, const void* 
                                void* rstd, int64_t rows, int64_t h, float eps, void* stream) {
     EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h <= 8192, EZL_EUNSUPPORTED,
                 "ezl_rmsnorm_fwd: need h %% 8 == 0 and h <= 8192 (got h=%lld)", (long long)h);
-    EZL_REQUIRE(x && weight && y && rstd, EZL_EINVAL, "ezl_rmsnorm_fwd: null pointer");
+    EZL_REQUIRE(rows == 0 || (x && weight && y && rstd), EZL_EINVAL, "ezl_rmsnorm_fwd: null pointer");
     EZL_REQUIRE((residual == nullptr) == (sum_out == nullptr), EZL_EINVAL,
                 "ezl_rmsnorm_fwd: residual and sum_out go together");
     EZL_REQUIRE(ezl_aligned16(x) && ezl_aligned16(weight) && ezl_aligned16(y) && ezl_aligned16(residual) &&
@@ -241,7 +241,7 @@ extern "C" int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight
                                void* workspace, int64_t workspace_bytes, int64_t rows, int64_t h, void* stream) {
     EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h <= 8192, EZL_EUNSUPPORTED,
                 "ezl_rmsnorm_bwd: need h %% 8 == 0 and h <= 8192 (got h=%lld)", (long long)h);
-    EZL_REQUIRE(dy && x && weight && rstd && dx && workspace, EZL_EINVAL, "ezl_rmsnorm_bwd: null pointer");
+    EZL_REQUIRE(weight && workspace && (rows == 0 || (dy && x && rstd && dx)), EZL_EINVAL, "ezl_rmsnorm_bwd: null pointer");
     EZL_REQUIRE((dw_bf16 != nullptr) != (dw_f32 != nullptr), EZL_EINVAL,
                 "ezl_rmsnorm_bwd: exactly one of dw_bf16 / dw_f32");
     EZL_REQUIRE(workspace_bytes >= ezl_rmsnorm_bwd_workspace_bytes(rows, h), EZL_EINVAL,

@@ -278,3 +278,45 @@ def test_ce_scale_by_scalar(K, gpu_device):
     assert torch.equal(x, y)
     K.scale_by_scalar_(y, torch.full((1,), 0.5, device=gpu_device))
     assert torch.equal(y.cpu(), (x.float().cpu() * 0.5).bfloat16())
+
+
+# ------------------------------------------------------------------------------------- empty inputs
+def test_empty_inputs_are_accepted_everywhere(K, gpu_device):
+    """Zero tokens (an empty micro-batch shard): every entry point returns empty results without launching on garbage."""
+    dev = gpu_device
+    h, f, V = 64, 96, 128
+    e = lambda *shape, dtype=torch.bfloat16: torch.empty(*shape, dtype=dtype, device=dev)  # noqa: E731
+    w = torch.ones(h, dtype=torch.bfloat16, device=dev)
+    y, rstd, _ = K.rmsnorm_fwd(e(0, h), w, 1e-6)
+    assert y.shape == (0, h) and rstd.numel() == 0
+    dx, dw = K.rmsnorm_bwd(e(0, h), e(0, h), w, rstd)
+    assert dx.shape == (0, h) and float(dw.float().abs().max()) == 0.0   # no rows: a zero weight gradient
+    assert K.swiglu_fwd(e(0, f), e(0, f)).numel() == 0
+    dg, du = K.swiglu_bwd(e(0, f), e(0, f), e(0, f))
+    assert dg.numel() == 0 and du.numel() == 0
+    assert K.add(e(0, h), e(0, h)).numel() == 0
+    assert K.transpose01(e(0, 2, h)).shape == (2, 0, h)
+    out, flag = K.embed_gather(torch.empty(1, 0, dtype=torch.int64, device=dev), torch.zeros(V, h, dtype=torch.bfloat16, device=dev))
+    assert out.shape == (1, 0, h) and flag.item() == 0
+    dW = torch.ones(V, h, dtype=torch.float32, device=dev)
+    K.embed_scatter_add(torch.empty(0, dtype=torch.int64, device=dev), e(0, h), dW)
+    assert float(dW.min()) == 1.0
+    wt = torch.zeros(f, h, dtype=torch.bfloat16, device=dev)
+    assert K.linear_fwd(e(0, h), wt).shape == (0, f)
+    assert K.linear_dgrad(e(0, f), wt).shape == (0, h)
+    gw = K.linear_wgrad(e(0, f), e(0, h))                               # K = 0 tokens: the gradient is exactly zero
+    assert gw.shape == (f, h) and float(gw.float().abs().max()) == 0.0
+    lg = e(0, V)
+    lb = torch.empty(0, dtype=torch.int64, device=dev)
+    wts, n = K.ce_prepare(lb, None)
+    assert float(n) == 0.0
+    loss_rows, grad = K.ce_fused(lg, lb, wts, n, inplace=False)
+    assert loss_rows.numel() == 0 and grad.numel() == 0
+    q, kv = e(0, 1, 4, 64), e(0, 1, 2, 64)
+    out, lse = K.attn_fwd(q, kv, kv)
+    assert out.shape == (0, 1, 4, 64) and lse.numel() == 0
+    dq, dk, dv = K.attn_bwd(q, kv, kv, out, e(0, 1, 4, 64), lse)
+    assert dq.numel() == 0 and dk.numel() == 0 and dv.numel() == 0
+    inv = 1.0 / (10000 ** (torch.arange(0, 64, 2, device=dev).float() / 64))
+    cos, sin = K.rope_table(inv, 8)
+    assert K.rope_apply(q, cos, sin).shape == (0, 1, 4, 64)
