@@ -67,6 +67,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="C2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--mode", choices=("graph", "eager"), default="graph",
+                    help="graph: the step is captured once into a HIP graph and replayed; eager: launched kernel by kernel")
     ap.add_argument("--no-optimizer-step", action="store_true", help="skip the separately timed AdamW + clipping step")
     ap.add_argument("--input-check", choices=("sync", "deferred"), default="deferred",
                     help="token-id range check of the embedding: blocking like the reference, or examined one call late")
@@ -104,8 +106,30 @@ def main():
         loss = step()
     functional.flush_input_checks()
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    elapsed_eager = time.perf_counter() - t0
     loss_value = float(loss.item())
+    elapsed = elapsed_eager
+    launch_mode = args.mode
+    if args.mode == "graph":
+        # the same kernels, captured once and replayed: no per-kernel host work, no launch gaps
+        try:
+            graphed = runner.GraphedStep(model, inputs, labels)
+        except Exception as exc:  # capture refused by the runtime: report the eager figures and say so
+            graphed = None
+            launch_mode = "eager (graph capture failed: %s)" % (str(exc).splitlines()[0][:120] if str(exc) else type(exc).__name__)
+            print("bench.py: %s" % launch_mode, file=sys.stderr)
+        if graphed is not None:
+            for _ in range(args.warmup):
+                graphed()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                loss = graphed()
+            graphed.flush()
+            torch.cuda.synchronize()
+            elapsed = time.perf_counter() - t0
+            assert float(loss.item()) == loss_value, "graph replay and eager step disagree"
+            del graphed
 
     # Second pass of the same K steps with every GEMM launch bracketed by two timing events on the launch stream.  The
     # events serialise the queue (about 20 us per launch), so they are kept out of the pass that `value` comes from.
@@ -130,7 +154,8 @@ def main():
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "%s: %s" % (args.workload, w["desc"]), "tokens_per_step": tokens_per_step,
                    "fp32_main_grads": True, "recomputed_layers": model.recompute_count,
-                   "input_id_check": args.input_check},
+                   "input_id_check": args.input_check, "launch": launch_mode,
+                   "eager_ms_per_step": round(elapsed_eager / args.steps * 1e3, 3)},
         "tflops": round(tflops, 1), "mfma_frac_end_to_end": round(tflops / PEAK_BF16_TFLOPS, 4), "loss": round(loss_value, 5),
         "roofline": {"kernel": "gemm_kernel (bf16 MFMA GEMM, %d launches/step)" % (len(timing) // max(args.steps, 1)),
                      "bound": "mfma", "achieved": round(gemm_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",

@@ -292,6 +292,7 @@ def _raise_for_id_flag(bad, ids, num_embeddings):
 # embedding call or flush_input_checks(); the launch queue never drains, the error surfaces one call late.
 _INPUT_CHECK = "sync"
 _PENDING_CHECKS = []
+CAPTURED_ID_FLAGS = []
 
 
 def set_input_check(mode):
@@ -315,6 +316,11 @@ def flush_input_checks(wait=True):
 def embedding(ids, weight):
     """Row gather; raises ValueError for an id >= vocab like the reference (:107-109)."""
     out, flag = EmbeddingFunction.apply(ids, weight)
+    if torch.cuda.is_current_stream_capturing():
+        # inside a graph capture nothing may synchronise: the flag tensor is handed to whoever captures
+        # (runner.GraphedStep), which reads it back after each replay
+        CAPTURED_ID_FLAGS.append((flag, weight.shape[0]))
+        return out
     if _INPUT_CHECK == "deferred":
         flush_input_checks(wait=False)
         host = torch.empty(1, dtype=torch.int32, pin_memory=True)
