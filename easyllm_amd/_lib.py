@@ -6,7 +6,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libezl.so")
+LIB_PATH = os.environ.get("EZL_LIBRARY") or os.path.join(_HERE, "lib", "libezl.so")  # EZL_LIBRARY: another build of the same ABI
 
 _vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
 _i64p = ctypes.POINTER(ctypes.c_int64)
