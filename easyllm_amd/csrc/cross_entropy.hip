@@ -67,9 +67,14 @@ __device__ __forceinline__ void row_max_sumexp(const T* __restrict__ xrow, T* __
         float f[8];
         Vec8<T>::load(xrow + i * 8, f);
         if (IN_LDS) Vec8<T>::store(srow + i * 8, f);
+        if (i * 8 + 8 <= vend) {  // whole vector inside [0, vend): no per-element compare
 #pragma unroll
-        for (int k = 0; k < 8; ++k)
-            if (i * 8 + k < vend) m = fmaxf(m, f[k]);
+            for (int k = 0; k < 8; ++k) m = fmaxf(m, f[k]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (i * 8 + k < vend) m = fmaxf(m, f[k]);
+        }
     }
     m = block_max(m, red);  // barriers inside also publish the staged row
     float s = 0.f;
@@ -77,9 +82,16 @@ __device__ __forceinline__ void row_max_sumexp(const T* __restrict__ xrow, T* __
     for (int i = threadIdx.x; i < v8; i += kCeBlock) {
         float f[8];
         Vec8<T>::load((IN_LDS ? (const T*)srow : xrow) + i * 8, f);
+        // the argument is never positive, so the bare instruction (no range fix-up) is exact enough: results below
+        // 2^-126 may flush to zero
+        if (i * 8 + 8 <= vend) {
 #pragma unroll
-        for (int k = 0; k < 8; ++k)
-            if (i * 8 + k < vend) s += exp2f(f[k] * kLog2e - mb);
+            for (int k = 0; k < 8; ++k) s += __builtin_amdgcn_exp2f(f[k] * kLog2e - mb);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (i * 8 + k < vend) s += __builtin_amdgcn_exp2f(f[k] * kLog2e - mb);
+        }
     }
     s = block_sum(s, red);
     m_out = m;
@@ -95,12 +107,17 @@ __device__ __forceinline__ void row_write_grad(const T* __restrict__ xrow, const
     for (int i = threadIdx.x; i < v8; i += kCeBlock) {
         float f[8];
         Vec8<T>::load((IN_LDS ? srow : xrow) + i * 8, f);
+        // columns past vend (cut_size) may exceed the row maximum, so this exp can overflow to +inf exactly as the
+        // reference's does; the bare instruction handles that range too
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            float p = exp2f(f[k] * kLog2e - lb);
-            if (i * 8 + k == target) p -= 1.0f;
-            f[k] = p * scale;
+        for (int k = 0; k < 8; ++k) f[k] = __builtin_amdgcn_exp2f(f[k] * kLog2e - lb);
+        if ((target >> 3) == i) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if ((target & 7) == k) f[k] -= 1.0f;
         }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) f[k] *= scale;
         Vec8<T>::store(grow + i * 8, f);
     }
 }
