@@ -179,6 +179,17 @@ def test_gemm_three_forms(K, gpu_device, T, n_in, n_out):
     close(mg, rdw, "gemm wgrad fp32 overwrite", rel=2e-3)
 
 
+def test_gemm_forward_with_unaligned_output_width(K, gpu_device):
+    """out features not a multiple of 4: the epilogue falls back from vector to element stores; K = 128 and 192 are the
+    shortest reductions of the direct-to-LDS kernel (2 and 3 K tiles), K = 64 goes through the register-staged one."""
+    for T, n_in, n_out in ((130, 128, 250), (257, 192, 31), (64, 64, 7)):
+        print("gemm odd width", T, n_in, n_out, flush=True)
+        x, w = rnd(T, n_in, seed=17), rnd(n_out, n_in, seed=18, scale=0.05)
+        y = K.linear_fwd(x.to(gpu_device), w.to(gpu_device))
+        assert tuple(y.shape) == (T, n_out)
+        close(y, x.float() @ w.float().t(), "gemm fwd odd width")
+
+
 def test_gemm_linearity_large(K, gpu_device):
     """Size-independent property at a full-size shape: (x1 + x2) W^T == x1 W^T + x2 W^T up to bf16
     rounding, and a column block of the result equals the GEMM on that block of W."""
