@@ -328,23 +328,54 @@ __global__ __launch_bounds__(kThreads) void attn_delta_kernel(AttnParams p) {
 // =================================================================================================
 // backward, dK and dV: a block owns 128 keys of one kv head and walks the queries at or after them
 // =================================================================================================
+// 8 waves: wave w works on keys 32 (w & 3) .. +31 and, of every 64-query tile, on the 32-query half (w >> 2); the two
+// waves that share a key group sit on the same SIMD, so the elementwise phase of one overlaps the MFMAs of the other.
+// To leave room for two waves per SIMD the K / V operand rows live in LDS (read as fragments per use) instead of in
+// registers; the two partial dK / dV of a key group are added through LDS at the end, always in the same order.
+constexpr int kDkdvThreads = 512;
+
 template <int D>
-__global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
+__global__ __launch_bounds__(kDkdvThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
     using TL = Tile<D>;
-    constexpr int STAGE = 2 * TL::ELEMS;                 // Q tile + dO tile
-    __shared__ __attribute__((aligned(16))) bf16_t smem[2 * STAGE];
-    __shared__ __attribute__((aligned(16))) float sstat[2][2][64];  // [stage][lse*log2e | delta][query]
+    constexpr int LD = TL::LD, CH = TL::CH;
+    constexpr int KV_ELEMS = 128 * LD;     // K (or V) rows of the block's 128 keys
+    constexpr int STAGE = 2 * TL::ELEMS;   // Q tile + dO tile, 64 rows each
+    constexpr int NCH_KV = 128 * CH / kDkdvThreads, NCH_Q = 64 * CH / kDkdvThreads;
+    __shared__ __attribute__((aligned(16))) bf16_t smem[2 * KV_ELEMS + 2 * STAGE];  // K V | (Q dO) x 2 stages
+    __shared__ __attribute__((aligned(16))) float sstat[2][2][64];                   // [stage][lse*log2e | delta][query]
+    static_assert(sizeof(bf16_t) * (2 * KV_ELEMS + 2 * STAGE) >= sizeof(float) * 4 * 2 * (D / 32) * 16 * 64,
+                  "the final reduction parks four waves' accumulators in the tile memory");
     int doc_start, doc_len, kbk;
     if (!find_block(p.cu, p.ndocs, p.s_len, p.T, blockIdx.x, 128, doc_start, doc_len, kbk)) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = wave & 3, half = wave >> 2;
     const int hk = blockIdx.y, group = p.nq / p.nk;
-    const int k0 = kbk * 128, kw0 = k0 + wave * 32;
+    const int k0 = kbk * 128, kw0 = k0 + kg * 32;
     const int tok_end = doc_start + doc_len;
     const int kj = kw0 + (lane & 31);  // this lane's key (document relative)
-    const int ktok = doc_start + (kj < doc_len ? kj : doc_len - 1);
-    bf16x8 kf[D / 16], vf[D / 16];
-    load_row_frags<D>(p.k + tok_off(ktok, p.s_len, p.k_ss, p.k_sb) + (int64_t)hk * D, lane, kf);
-    load_row_frags<D>(p.v + tok_off(ktok, p.s_len, p.v_ss, p.v_sb) + (int64_t)hk * D, lane, vf);
+    bf16_t* sK = smem;
+    bf16_t* sV = smem + KV_ELEMS;
+    bf16_t* sQ0 = smem + 2 * KV_ELEMS;
+
+    {   // K / V rows of the block: rows past the document's end re-read its last row (always masked)
+        const bf16_t* kdoc = p.k + tok_off(doc_start, p.s_len, p.k_ss, p.k_sb) + (int64_t)hk * D;
+        const bf16_t* vdoc = p.v + tok_off(doc_start, p.s_len, p.v_ss, p.v_sb) + (int64_t)hk * D;
+        bf16x8 rk[NCH_KV], rv[NCH_KV];
+#pragma unroll
+        for (int i = 0; i < NCH_KV; ++i) {
+            const int c = tid + kDkdvThreads * i;
+            int n = k0 + c / CH;
+            n = n < doc_len ? n : doc_len - 1;
+            rk[i] = *reinterpret_cast<const bf16x8*>(kdoc + (int64_t)n * p.k_ss + (c % CH) * 8);
+            rv[i] = *reinterpret_cast<const bf16x8*>(vdoc + (int64_t)n * p.v_ss + (c % CH) * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < NCH_KV; ++i) {
+            const int c = tid + kDkdvThreads * i;
+            *reinterpret_cast<bf16x8*>(sK + (c / CH) * LD + (c % CH) * 8) = rk[i];
+            *reinterpret_cast<bf16x8*>(sV + (c / CH) * LD + (c % CH) * 8) = rv[i];
+        }
+    }
 
     f32x16 dkacc[D / 32], dvacc[D / 32];
 #pragma unroll
@@ -359,13 +390,19 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
 
     const bf16_t* qdoc = p.q + tok_off(doc_start, p.s_len, p.q_ss, p.q_sb);
     const bf16_t* dodoc = p.dout + tok_off(doc_start, p.s_len, p.do_ss, p.do_sb);
-    bf16x8 rq[TL::NCH], rdo[TL::NCH];
+    bf16x8 rq[NCH_Q], rdo[NCH_Q];
     float rstat = 0.f;  // threads 0..63: lse*log2e of query tid; 64..127: delta of query tid-64
     auto load_iter = [&](int it) {
         const int hq = hk * group + it / nqt;
         const int row0 = (qt0 + it % nqt) * 64;
-        TL::load(qdoc + (int64_t)hq * D, p.q_ss, row0, doc_len, tid, rq);
-        TL::load(dodoc + (int64_t)hq * D, p.do_ss, row0, doc_len, tid, rdo);
+#pragma unroll
+        for (int i = 0; i < NCH_Q; ++i) {
+            const int c = tid + kDkdvThreads * i;
+            int n = row0 + c / CH;
+            n = n < doc_len ? n : doc_len - 1;
+            rq[i] = *reinterpret_cast<const bf16x8*>(qdoc + (int64_t)hq * D + (int64_t)n * p.q_ss + (c % CH) * 8);
+            rdo[i] = *reinterpret_cast<const bf16x8*>(dodoc + (int64_t)hq * D + (int64_t)n * p.do_ss + (c % CH) * 8);
+        }
         if (tid < 128) {
             const int n = doc_start + row0 + (tid & 63);
             rstat = 0.f;
@@ -373,55 +410,53 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
         }
     };
     auto store_iter = [&](int stage) {
-        TL::store(smem + stage * STAGE, tid, rq);
-        TL::store(smem + stage * STAGE + TL::ELEMS, tid, rdo);
+        bf16_t* sq = sQ0 + stage * STAGE;
+#pragma unroll
+        for (int i = 0; i < NCH_Q; ++i) {
+            const int c = tid + kDkdvThreads * i;
+            *reinterpret_cast<bf16x8*>(sq + (c / CH) * LD + (c % CH) * 8) = rq[i];
+            *reinterpret_cast<bf16x8*>(sq + TL::ELEMS + (c / CH) * LD + (c % CH) * 8) = rdo[i];
+        }
         if (tid < 128) sstat[stage][tid >> 6][tid & 63] = rstat;
     };
     load_iter(0);
     store_iter(0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K/V rows held in registers have landed (see the forward kernel)
     if (total > 1) load_iter(1);
     __syncthreads();
 
     for (int it = 0; it < total; ++it) {
         const int cur = it & 1;
-        const bf16_t* sQ = smem + cur * STAGE;
+        const bf16_t* sQ = sQ0 + cur * STAGE;
         const bf16_t* sdO = sQ + TL::ELEMS;
         if (it + 1 < total) store_iter(cur ^ 1);
         if (it + 2 < total) load_iter(it + 2);
         const int qbase = (qt0 + it % nqt) * 64;
-#pragma unroll
-        for (int sub = 0; sub < 2; ++sub) {
-            const int qs0 = qbase + sub * 32;
-            if (qs0 + 31 < kw0 || qs0 >= doc_len) continue;  // all queries before this wave's keys / past the end
-            // S = Q K^T and dP = dO V^T in groups of 2 d-steps; the next group's fragments are in flight meanwhile
-            constexpr int NG = D / 32;
+        const int qs0 = qbase + half * 32;
+        if (!(qs0 + 31 < kw0 || qs0 >= doc_len)) {  // else: all queries before this wave's keys / past the end
+            // S = Q K^T and dP = dO V^T, one d-step (4 fragments, 2 MFMAs) at a time with the next step's fragments in flight
+            constexpr int NS = D / 16;
             f32x16 sacc, dpacc;
-            bf16x8 fq[2][2], fo[2][2];
-            auto ldqo = [&](int g, int buf) {
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    fq[buf][i] = TL::frag_kc(sQ, sub * 32, g * 2 + i, lane);
-                    fo[buf][i] = TL::frag_kc(sdO, sub * 32, g * 2 + i, lane);
-                }
+            bf16x8 fq[2], fo[2], fk[2], fv[2];
+            auto lda = [&](int g, int buf) {
+                fq[buf] = TL::frag_kc(sQ, half * 32, g, lane);
+                fk[buf] = TL::frag_kc(sK, kg * 32, g, lane);
+                fo[buf] = TL::frag_kc(sdO, half * 32, g, lane);
+                fv[buf] = TL::frag_kc(sV, kg * 32, g, lane);
             };
-            ldqo(0, 0);
+            lda(0, 0);
 #pragma unroll
             for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                if (g + 1 < NG) ldqo(g + 1, (g + 1) & 1);
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[g & 1][i], kf[g * 2 + i], sacc, 0, 0, 0);
-                    dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fo[g & 1][i], vf[g * 2 + i], dpacc, 0, 0, 0);
-                }
+            for (int g = 0; g < NS; ++g) {
+                if (g + 1 < NS) lda(g + 1, (g + 1) & 1);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[g & 1], fk[g & 1], sacc, 0, 0, 0);
+                dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fo[g & 1], fv[g & 1], dpacc, 0, 0, 0);
             }
             __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                if (g + 1 < NG) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+            for (int g = 0; g < NS; ++g) {
+                if (g + 1 < NS) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
             }
             // dO^T / Q^T fragments, two d blocks at a time; the first pair's latency hides under the elementwise math
             constexpr int NT = 2 * (D / 64);  // (16-query step, d-block pair) groups
@@ -430,22 +465,22 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
                 const int tt = gt / (D / 64), dbp = gt % (D / 64);
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
-                    fto[buf][i] = TL::frag_tr(sdO, sub * 32 + 16 * tt, (2 * dbp + i) * 32, lane);
-                    ftq[buf][i] = TL::frag_tr(sQ, sub * 32 + 16 * tt, (2 * dbp + i) * 32, lane);
+                    fto[buf][i] = TL::frag_tr(sdO, half * 32 + 16 * tt, (2 * dbp + i) * 32, lane);
+                    ftq[buf][i] = TL::frag_tr(sQ, half * 32 + 16 * tt, (2 * dbp + i) * 32, lane);
                 }
             };
             ldt(0, 0);
             // accumulator register r <-> query qs0 + acc_row(r); lane <-> key kj
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-                const int ql = sub * 32 + 8 * r4 + 4 * (lane >> 5);
+                const int ql = half * 32 + 8 * r4 + 4 * (lane >> 5);
                 const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sstat[cur][0][ql]);
                 const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sstat[cur][1][ql]);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int r = r4 * 4 + e;
                     const int qidx = qbase + ql + e;
-                    float pe = __builtin_amdgcn_exp2f(sacc[r] * sl2 - l4[e]);
+                    float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], sl2, -l4[e]));
                     if (kj > qidx || qidx >= doc_len) pe = 0.f;
                     sacc[r] = pe;
                     dpacc[r] = pe * (dpacc[r] - d4[e]);
@@ -466,7 +501,21 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
         }
         __syncthreads();
     }
-    if (kj < doc_len) {
+
+    // fold the two halves of every key group: waves 4..7 park their accumulators in LDS (32 KiB each, lane-contiguous),
+    // waves 0..3 add them to their own and write the rows out
+    float* red = reinterpret_cast<float*>(smem) + (size_t)kg * (2 * (D / 32) * 16 * 64);
+    if (half == 1) {
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                red[(db * 16 + r) * 64 + lane] = dkacc[db][r];
+                red[((D / 32 + db) * 16 + r) * 64 + lane] = dvacc[db][r];
+            }
+    }
+    __syncthreads();
+    if (half == 0 && kj < doc_len) {
         bf16_t* dkrow = p.dk + tok_off(doc_start + kj, p.s_len, p.dk_ss, p.dk_sb) + (int64_t)hk * D;
         bf16_t* dvrow = p.dv + tok_off(doc_start + kj, p.s_len, p.dv_ss, p.dv_sb) + (int64_t)hk * D;
 #pragma unroll
@@ -476,8 +525,9 @@ __global__ __launch_bounds__(kThreads) void attn_bwd_dkdv_kernel(AttnParams p) {
                 bf16x4 a, b;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    a[e] = (bf16_t)(dkacc[db][r4 * 4 + e] * p.scale);
-                    b[e] = (bf16_t)dvacc[db][r4 * 4 + e];
+                    const int r = r4 * 4 + e;
+                    a[e] = (bf16_t)((dkacc[db][r] + red[(db * 16 + r) * 64 + lane]) * p.scale);
+                    b[e] = (bf16_t)(dvacc[db][r] + red[((D / 32 + db) * 16 + r) * 64 + lane]);
                 }
                 const int dcol = db * 32 + 8 * r4 + 4 * (lane >> 5);
                 *reinterpret_cast<bf16x4*>(dkrow + dcol) = a;
@@ -684,11 +734,11 @@ extern "C" int ezl_attn_bwd(const void* q, const void* k, const void* v, const v
     const dim3 gridk((unsigned)((total_tokens + 127) / 128 + ndocs + total_tokens / s_len), (unsigned)nk);
     if (d == 128) {
         hipLaunchKernelGGL(attn_delta_kernel<128>, dim3((unsigned)g), dim3(kThreads), 0, st, p);
-        hipLaunchKernelGGL(attn_bwd_dkdv_kernel<128>, gridk, dim3(kThreads), 0, st, p);
+        hipLaunchKernelGGL(attn_bwd_dkdv_kernel<128>, gridk, dim3(kDkdvThreads), 0, st, p);
         hipLaunchKernelGGL(attn_bwd_dq_kernel<128>, gridq, dim3(kThreads), 0, st, p);
     } else {
         hipLaunchKernelGGL(attn_delta_kernel<64>, dim3((unsigned)g), dim3(kThreads), 0, st, p);
-        hipLaunchKernelGGL(attn_bwd_dkdv_kernel<64>, gridk, dim3(kThreads), 0, st, p);
+        hipLaunchKernelGGL(attn_bwd_dkdv_kernel<64>, gridk, dim3(kDkdvThreads), 0, st, p);
         hipLaunchKernelGGL(attn_bwd_dq_kernel<64>, gridq, dim3(kThreads), 0, st, p);
     }
     EZL_LAUNCH_CHECK("ezl_attn_bwd");
