@@ -17,7 +17,8 @@ against library routines, closed forms and invariants:
   attention ............ pinned (``F.scaled_dot_product_attention`` causal + GQA, per-document split,
                                 brute-force python loops on tiny inputs)
   swiglu ............... pinned (``F.silu``, closed-form derivative vs autograd)
-  layer / model wiring . pinned (``transformers.LlamaForCausalLM`` built from a local config)
+  layer / model wiring . pinned (``transformers.LlamaForCausalLM`` built from a local config, live and through the
+                                committed fixture tests/golden/hf_llama_tiny.npz: loss, logits, every gradient)
   cross entropy ........ pinned (``F.cross_entropy``, uniform-logits ln V, shift invariance)
   dynamic-ckpt rule .... pinned (table-driven known answers written from the reference text)
   packed inputs ........ pinned (hand-worked known answers)
