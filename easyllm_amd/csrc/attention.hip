@@ -75,6 +75,21 @@ __device__ __forceinline__ bool find_block(const int* __restrict__ cu, int ndocs
     return false;
 }
 
+// The hardware deals consecutive workgroups (x fastest, then y) round-robin to the 8 XCDs, each with an L2 of its own.
+// With the plain (block, head) numbering every XCD would touch the K / V rows of every head and its L2 would keep missing;
+// renumbered, an XCD gets whole heads, a few at a time.  by: head, bx: block index inside the head's token blocks.
+__device__ __forceinline__ void xcd_head_blocks(int nheads, int& bx, int& by) {
+    bx = blockIdx.x;
+    by = blockIdx.y;
+    if ((nheads & 7) == 0) {
+        const int gx = gridDim.x;
+        const int lin = blockIdx.y * gx + blockIdx.x;
+        const int idx = lin >> 3;
+        by = (lin & 7) * (nheads >> 3) + idx / gx;
+        bx = idx % gx;
+    }
+}
+
 template <int D>
 struct Tile {
     static constexpr int LD = D + 24;             // padded row stride in elements
@@ -152,10 +167,12 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
     using TL = Tile<D>;
     __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS];  // K0 V0 K1 V1
     int doc_start, doc_len, qb;
-    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, blockIdx.x, 128, doc_start, doc_len, qb)) return;
+    int bx, by;
+    xcd_head_blocks(p.nq, bx, by);
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;
     qb = (doc_len + 127) / 128 - 1 - qb;  // longest rows first
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int hq = blockIdx.y, hk = hq / (p.nq / p.nk);
+    const int hq = by, hk = hq / (p.nq / p.nk);
     const int q0 = qb * 128, qw0 = q0 + wave * 32;
     const int tok_end = doc_start + doc_len;
     const int qi = qw0 + (lane & 31);                        // this lane's query (document relative)
@@ -346,10 +363,12 @@ __global__ __launch_bounds__(kDkdvThreads) void attn_bwd_dkdv_kernel(AttnParams 
     static_assert(sizeof(bf16_t) * (2 * KV_ELEMS + 2 * STAGE) >= sizeof(float) * 4 * 2 * (D / 32) * 16 * 64,
                   "the final reduction parks four waves' accumulators in the tile memory");
     int doc_start, doc_len, kbk;
-    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, blockIdx.x, 128, doc_start, doc_len, kbk)) return;
+    int bx, by;
+    xcd_head_blocks(p.nk, bx, by);
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, kbk)) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kg = wave & 3, half = wave >> 2;
-    const int hk = blockIdx.y, group = p.nq / p.nk;
+    const int hk = by, group = p.nq / p.nk;
     const int k0 = kbk * 128, kw0 = k0 + kg * 32;
     const int tok_end = doc_start + doc_len;
     const int kj = kw0 + (lane & 31);  // this lane's key (document relative)
@@ -544,10 +563,12 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
     using TL = Tile<D>;
     __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS];  // K0 V0 K1 V1
     int doc_start, doc_len, qb;
-    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, blockIdx.x, 128, doc_start, doc_len, qb)) return;
+    int bx, by;
+    xcd_head_blocks(p.nq, bx, by);
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;
     qb = (doc_len + 127) / 128 - 1 - qb;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int hq = blockIdx.y, hk = hq / (p.nq / p.nk);
+    const int hq = by, hk = hq / (p.nq / p.nk);
     const int q0 = qb * 128, qw0 = q0 + wave * 32;
     const int tok_end = doc_start + doc_len;
     const int qi = qw0 + (lane & 31);
