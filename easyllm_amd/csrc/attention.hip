@@ -29,6 +29,8 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
 typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(1))) const void gvoid;
 
 struct AttnParams {
     const bf16_t* q; const bf16_t* k; const bf16_t* v; const bf16_t* o; const bf16_t* dout;
@@ -95,28 +97,42 @@ struct Tile {
     static constexpr int LD = D + 24;             // padded row stride in elements
     static constexpr int CH = D / 8;              // 128-bit chunks per row
     static constexpr int ROWS = 64;
-    static constexpr int NCH = ROWS * CH / kThreads;  // chunks per thread
     static constexpr int ELEMS = ROWS * LD;
 
-    // rows row0 .. row0+63 of a document whose token 0 (head column included) is at `base`; rows at or past
-    // doc_len re-read the document's last row: finite values that only ever meet masked (zero) probabilities
-    static __device__ __forceinline__ void load(const bf16_t* __restrict__ base, int64_t ss, int row0, int doc_len, int tid,
-                                                bf16x8* r) {
+    // ---- tile rows straight from global memory into LDS (global_load_lds, 16 bytes per lane) ----
+    // One wave instruction fills 1 KiB of consecutive LDS, i.e. 1024 / (2 LD) padded rows: instruction q of a tile covers
+    // bytes 1024 q .. 1024 q + 1023 of its LDS image, and the lane that falls on row padding re-reads the row's first chunk.
+    // Rows at or past the document's end re-read its last row: finite values that only ever meet masked probabilities.
+    // NWAVES waves share the NQ instructions of a tile: wave w issues q = w, w + NWAVES, ...
+    static constexpr int NQ = (ROWS * LD * 2 + 1023) / 1024;
+    static_assert(ROWS * LD * 2 % 1024 == 0, "a tile is a whole number of 1 KiB pieces");
+    template <int NWAVES>
+    struct Direct {
+        static constexpr int NJ = (NQ + NWAVES - 1) / NWAVES;
+        uint32_t off[NJ];  // global byte offset of this lane's chunk from the tile's first row, per instruction
+        // last: last valid row of the tile (63, or fewer in a document's ragged last tile: later rows re-read it)
+        __device__ __forceinline__ void init(int64_t ss, int lane, int wave, int last) {
 #pragma unroll
-        for (int i = 0; i < NCH; ++i) {
-            const int c = tid + kThreads * i;
-            int n = row0 + c / CH;
-            n = n < doc_len ? n : doc_len - 1;
-            r[i] = *reinterpret_cast<const bf16x8*>(base + (int64_t)n * ss + (c % CH) * 8);
+            for (int j = 0; j < NJ; ++j) {
+                const int q = wave + NWAVES * j;
+                const int byte = q * 1024 + lane * 16;
+                int row = byte / (LD * 2);
+                int colb = byte - row * (LD * 2);
+                colb = colb < D * 2 ? colb : 0;
+                row = row < last ? row : last;
+                off[j] = (uint32_t)row * (uint32_t)(ss * 2) + (uint32_t)colb;
+            }
         }
-    }
-    static __device__ __forceinline__ void store(bf16_t* __restrict__ s, int tid, const bf16x8* r) {
+        // tile_rows: global address of the tile's first row (head column included); stage: its LDS image
+        __device__ __forceinline__ void issue(const bf16_t* tile_rows, bf16_t* stage, int wave) const {
+            const char* g = reinterpret_cast<const char*>(tile_rows);
 #pragma unroll
-        for (int i = 0; i < NCH; ++i) {
-            const int c = tid + kThreads * i;
-            *reinterpret_cast<bf16x8*>(s + (c / CH) * LD + (c % CH) * 8) = r[i];
+            for (int j = 0; j < NJ; ++j) {
+                const int q = wave + NWAVES * j;
+                if (q < NQ) __builtin_amdgcn_global_load_lds((gvoid*)(g + off[j]), (lds_void*)(stage + q * 512), 16, 0, 0);
+            }
         }
-    }
+    };
     // operand whose k index is d:   lane -> row (row0 + lane&31), d = kd*16 + 8*(lane>>5) ..+7
     static __device__ __forceinline__ bf16x8 frag_kc(const bf16_t* __restrict__ s, int row0, int kd, int lane) {
         return *reinterpret_cast<const bf16x8*>(s + (row0 + (lane & 31)) * LD + kd * 16 + (lane >> 5) * 8);
@@ -171,7 +187,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
     xcd_head_blocks(p.nq, bx, by);
     if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;
     qb = (doc_len + 127) / 128 - 1 - qb;  // longest rows first
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hq = by, hk = hq / (p.nq / p.nk);
     const int q0 = qb * 128, qw0 = q0 + wave * 32;
     const int tok_end = doc_start + doc_len;
@@ -185,18 +201,27 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
     const int64_t kh = (int64_t)hk * D;
     const bf16_t* kbase = p.k + tok_off(doc_start, p.s_len, p.k_ss, p.k_sb) + kh;
     const bf16_t* vbase = p.v + tok_off(doc_start, p.s_len, p.v_ss, p.v_sb) + kh;
-    bf16x8 rk[TL::NCH], rv[TL::NCH];
-    TL::load(kbase, p.k_ss, 0, doc_len, tid, rk);
-    TL::load(vbase, p.v_ss, 0, doc_len, tid, rv);
-    TL::store(smem, tid, rk);
-    TL::store(smem + TL::ELEMS, tid, rv);
-    // every load issued so far (the per-lane operand rows included) has landed before the loop starts;
-    // otherwise their first use inside the loop would also wait for the tile loads issued just before it
+    // K / V tiles go from global memory straight into LDS, one tile ahead of the one being worked on
+    typename TL::template Direct<kThreads / 64> kld, vld;
+    kld.init(p.k_ss, lane, wave, 63);
+    vld.init(p.v_ss, lane, wave, 63);
+    auto issue_tile = [&](int t, int stage) {
+        const int row0 = t * 64;
+        bf16_t* sk = smem + stage * 2 * TL::ELEMS;
+        if (row0 + 64 <= doc_len) {
+            kld.issue(kbase + (int64_t)row0 * p.k_ss, sk, wave);
+            vld.issue(vbase + (int64_t)row0 * p.v_ss, sk + TL::ELEMS, wave);
+        } else {  // the document's ragged last tile: rows past its end re-read its last row
+            typename TL::template Direct<kThreads / 64> ke, ve;
+            ke.init(p.k_ss, lane, wave, doc_len - 1 - row0);
+            ve.init(p.v_ss, lane, wave, doc_len - 1 - row0);
+            ke.issue(kbase + (int64_t)row0 * p.k_ss, sk, wave);
+            ve.issue(vbase + (int64_t)row0 * p.v_ss, sk + TL::ELEMS, wave);
+        }
+    };
+    issue_tile(0, 0);
+    // every load issued so far (the per-lane operand rows included) has landed before the loop starts
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    if (ntiles > 1) {
-        TL::load(kbase, p.k_ss, 64, doc_len, tid, rk);
-        TL::load(vbase, p.v_ss, 64, doc_len, tid, rv);
-    }
     __syncthreads();
 
     f32x16 oacc[D / 32];
@@ -211,14 +236,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
         const int cur = t & 1;
         const bf16_t* sK = smem + cur * 2 * TL::ELEMS;
         const bf16_t* sV = sK + TL::ELEMS;
-        if (t + 1 < ntiles) {
-            TL::store(smem + (cur ^ 1) * 2 * TL::ELEMS, tid, rk);
-            TL::store(smem + (cur ^ 1) * 2 * TL::ELEMS + TL::ELEMS, tid, rv);
-        }
-        if (t + 2 < ntiles) {
-            TL::load(kbase, p.k_ss, (t + 2) * 64, doc_len, tid, rk);
-            TL::load(vbase, p.v_ss, (t + 2) * 64, doc_len, tid, rv);
-        }
+        if (t + 1 < ntiles) issue_tile(t + 1, cur ^ 1);  // that stage was last read before the barrier that ended tile t-1
         const int key0 = t * 64;
         if (key0 <= qw0 + 31) {  // otherwise every key of the tile is after every query of this wave
             // S^T = K Q^T in groups of 4 MFMAs; the K fragments of the next group are in flight meanwhile
@@ -300,6 +318,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
                     oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv[g & 1][db], pf, oacc[db], 0, 0, 0);
             }
         }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of the next tile are in LDS
         __syncthreads();
     }
     const float ltot = lsum + __shfl_xor(lsum, 32, 64);
@@ -567,7 +586,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
     xcd_head_blocks(p.nq, bx, by);
     if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;
     qb = (doc_len + 127) / 128 - 1 - qb;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hq = by, hk = hq / (p.nq / p.nk);
     const int q0 = qb * 128, qw0 = q0 + wave * 32;
     const int tok_end = doc_start + doc_len;
@@ -584,18 +603,27 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
     const int64_t kh = (int64_t)hk * D;
     const bf16_t* kbase = p.k + tok_off(doc_start, p.s_len, p.k_ss, p.k_sb) + kh;
     const bf16_t* vbase = p.v + tok_off(doc_start, p.s_len, p.v_ss, p.v_sb) + kh;
-    bf16x8 rk[TL::NCH], rv[TL::NCH];
-    TL::load(kbase, p.k_ss, 0, doc_len, tid, rk);
-    TL::load(vbase, p.v_ss, 0, doc_len, tid, rv);
-    TL::store(smem, tid, rk);
-    TL::store(smem + TL::ELEMS, tid, rv);
-    // every load issued so far (the per-lane operand rows included) has landed before the loop starts;
-    // otherwise their first use inside the loop would also wait for the tile loads issued just before it
+    // K / V tiles go from global memory straight into LDS, one tile ahead of the one being worked on
+    typename TL::template Direct<kThreads / 64> kld, vld;
+    kld.init(p.k_ss, lane, wave, 63);
+    vld.init(p.v_ss, lane, wave, 63);
+    auto issue_tile = [&](int t, int stage) {
+        const int row0 = t * 64;
+        bf16_t* sk = smem + stage * 2 * TL::ELEMS;
+        if (row0 + 64 <= doc_len) {
+            kld.issue(kbase + (int64_t)row0 * p.k_ss, sk, wave);
+            vld.issue(vbase + (int64_t)row0 * p.v_ss, sk + TL::ELEMS, wave);
+        } else {  // the document's ragged last tile: rows past its end re-read its last row
+            typename TL::template Direct<kThreads / 64> ke, ve;
+            ke.init(p.k_ss, lane, wave, doc_len - 1 - row0);
+            ve.init(p.v_ss, lane, wave, doc_len - 1 - row0);
+            ke.issue(kbase + (int64_t)row0 * p.k_ss, sk, wave);
+            ve.issue(vbase + (int64_t)row0 * p.v_ss, sk + TL::ELEMS, wave);
+        }
+    };
+    issue_tile(0, 0);
+    // every load issued so far (the per-lane operand rows included) has landed before the loop starts
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    if (ntiles > 1) {
-        TL::load(kbase, p.k_ss, 64, doc_len, tid, rk);
-        TL::load(vbase, p.v_ss, 64, doc_len, tid, rv);
-    }
     __syncthreads();
 
     f32x16 dqacc[D / 32];
@@ -609,14 +637,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
         const int cur = t & 1;
         const bf16_t* sK = smem + cur * 2 * TL::ELEMS;
         const bf16_t* sV = sK + TL::ELEMS;
-        if (t + 1 < ntiles) {
-            TL::store(smem + (cur ^ 1) * 2 * TL::ELEMS, tid, rk);
-            TL::store(smem + (cur ^ 1) * 2 * TL::ELEMS + TL::ELEMS, tid, rv);
-        }
-        if (t + 2 < ntiles) {
-            TL::load(kbase, p.k_ss, (t + 2) * 64, doc_len, tid, rk);
-            TL::load(vbase, p.v_ss, (t + 2) * 64, doc_len, tid, rv);
-        }
+        if (t + 1 < ntiles) issue_tile(t + 1, cur ^ 1);  // that stage was last read before the barrier that ended tile t-1
         const int key0 = t * 64;
         if (key0 <= qw0 + 31) {
             const bool on_diag = key0 + 63 > qw0;
@@ -675,6 +696,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
                 }
             }
         }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of the next tile are in LDS
         __syncthreads();
     }
     if (qi < doc_len) {
