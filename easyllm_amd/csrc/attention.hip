@@ -231,6 +231,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
         for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
     float m = -INFINITY, lsum = 0.f;
     const float sl2 = p.scale * kLog2e;
+    const float tau = 8.0f / sl2;  // 2^8 in units of the raw scores
 
     for (int t = 0; t < ntiles; ++t) {
         const int cur = t & 1;
@@ -287,8 +288,20 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, sacc[kb][r]);
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-            const float mnew = fmaxf(m, mloc);
-            const float moff = (mnew == -INFINITY ? 0.f : mnew) * sl2;
+            // The reference point m of the exponentials only has to bound them, not equal the running maximum: it is moved
+            // (and O, l rescaled) only when some row of the wave has outgrown it by more than a factor 2^8, which after
+            // the first tiles is rare.  Probabilities then reach at most 2^8 before the final division by l.
+            if (__builtin_amdgcn_ballot_w64(mloc > m + tau) != 0) {
+                const float mnew = fmaxf(m, mloc);
+                const float alpha = __builtin_amdgcn_exp2f((m - (mnew == -INFINITY ? 0.f : mnew)) * sl2);  // m = -inf: 0
+                lsum *= alpha;
+#pragma unroll
+                for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+                m = mnew;
+            }
+            const float moff = (m == -INFINITY ? 0.f : m) * sl2;
             float psum = 0.f;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
@@ -298,16 +311,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
                     sacc[kb][r] = pe;
                     psum += pe;
                 }
-            if (__builtin_amdgcn_ballot_w64(mnew > m) != 0) {  // some query of this wave saw a new maximum
-                const float alpha = __builtin_amdgcn_exp2f(__builtin_fmaf(m, sl2, -moff));
-                lsum *= alpha;
-#pragma unroll
-                for (int i = 0; i < D / 32; ++i)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
-            }
             lsum += psum;
-            m = mnew;
             // O^T += V^T P^T, 4 groups of (16 keys x all d blocks)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {

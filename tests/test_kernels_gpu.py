@@ -239,6 +239,31 @@ def test_attention_varlen_across_batch_rows(K, gpu_device):
     _attn_case(K, gpu_device, 256, 2, 4, 4, 128, cu, 40)
 
 
+def test_attention_forward_with_drifting_and_jumping_maxima(K, gpu_device):
+    """The forward kernel moves the reference point of its exponentials only when a row's maximum has outgrown it by a
+    factor 2^8.  Scores here grow along the keys: slowly for most rows (many tiles pass between two moves, probabilities
+    far above 1 in between), in jumps for the keys after position 700; output and logsumexp against the oracle in fp32."""
+    s, nq, d = 1024, 2, 128
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn(s, 1, nq, d, generator=g) * 0.3 + 1.0
+    ramp = torch.linspace(0.2, 2.2, s).view(s, 1, 1, 1)
+    k = torch.randn(s, 1, nq, d, generator=g) * 0.3 + ramp * 0.5
+    k[700:] *= 1.8
+    v = torch.randn(s, 1, nq, d, generator=g)
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    scores = torch.einsum("qhd,khd->hqk", q[:, 0].float(), k[:, 0].float()) / d ** 0.5
+    scores = scores.masked_fill(torch.triu(torch.ones(s, s, dtype=torch.bool), 1), float("-inf"))
+    # the case is what the docstring says: row maxima keep rising, by more than 2^8 in total
+    run_max = scores.cummax(-1).values
+    rise = (run_max[..., -1] - run_max[..., 64]) * 1.4427  # in powers of two
+    assert rise[:, 768:].min() > 16 and 2 < rise[:, 300:700].min() and rise[:, 300:700].max() < 16
+    ref_lse = torch.logsumexp(scores, -1)
+    ref = torch.einsum("hqk,khd->qhd", torch.softmax(scores, -1), v[:, 0].float())
+    out, lse = K.attn_fwd(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), None)
+    close(out[:, 0], ref, "attn out (rising maxima)")
+    assert torch.allclose(lse.cpu().view(nq, s), ref_lse, rtol=1e-4, atol=2e-3)
+
+
 # ------------------------------------------------------------------------------------- cross entropy
 @pytest.mark.parametrize("rows,V,dtype,cut", [(33, 32000, torch.bfloat16, 0), (5, 152064, torch.bfloat16, 0),
                                               (17, 4096, torch.float32, 0), (9, 32000, torch.float32, 0),
