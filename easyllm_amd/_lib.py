@@ -10,6 +10,7 @@ LIB_PATH = os.environ.get("EZL_LIBRARY") or os.path.join(_HERE, "lib", "libezl.s
 
 _vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
 _i64p = ctypes.POINTER(ctypes.c_int64)
+_vpp = ctypes.POINTER(ctypes.c_void_p)
 
 # name -> argtypes; the single source of truth for the symbol table on the Python side
 SIGNATURES = {
@@ -28,6 +29,7 @@ SIGNATURES = {
     "ezl_bias_add": [_vp, _vp, _vp, _i64, _i64, _vp],
     "ezl_bias_grad": [_vp, _vp, _vp, _i32, _vp, _i64, _i64, _i64, _vp],
     "ezl_gemm_bf16": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
+    "ezl_gemm_bf16_ksplit": [_i32, _vpp, _vpp, _vp, _i64, _i64, _i64p, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
     "ezl_attn_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64p, _vp],
     "ezl_attn_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32,
                      _i64p, _vp],

@@ -327,10 +327,23 @@ template <> struct Out4<float> { typedef f32x4 type; };
 // used because it sustains a higher clock than 32x32x16 under the board's power limit (fewer accumulator-register
 // accesses per flop).  A 64-wide K tile is worked off in four phases (k half, M half): a phase issues 16 MFMAs on 4 A and
 // 4 B fragments while the fragments of the next phase are read from LDS into the other register set.
-template <bool A_KC, bool B_KC, typename OutT>
+//
+// MULTI: the reduction runs over up to three (A, B) pairs in turn, C (=|+=) A0 B0 + A1 B1 + A2 B2, all pairs with the same
+// leading dimensions: the input gradient of several linears that share their input (q / k / v, gate / up) in one launch,
+// summed in fp32, instead of one launch per pair that reads and rewrites the bf16 result.  K is the total reduction
+// length; pair 1 starts at K tile t1, pair 2 at t2 (INT_MAX when absent).
+struct KSegments {
+    const bf16_t* A1;
+    const bf16_t* B1;
+    const bf16_t* A2;
+    const bf16_t* B2;
+    int t1, t2;
+};
+
+template <bool A_KC, bool B_KC, typename OutT, bool MULTI = false>
 __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B, OutT* __restrict__ C,
                                                        int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
-                                                       int tiles_m, int tiles_n) {
+                                                       int tiles_m, int tiles_n, const KSegments seg = KSegments()) {
     constexpr int NW = 8, WAVES_N = 4;
     __shared__ __attribute__((aligned(1024))) bf16_t smem[4 * DTILE];  // A0 B0 A1 B1
     const int tid = threadIdx.x, lane = tid & 63;
@@ -389,8 +402,16 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
                 acc[half * 4 + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[bbuf][j], fa[abuf][i], acc[half * 4 + i][j], 0, 0, 0);
     };
     auto issue_tile = [&](int t, int stage) {
-        la.issue(A + (int64_t)t * astep, smem + stage * 2 * DTILE, wave);
-        lb.issue(B + (int64_t)t * bstep, smem + stage * 2 * DTILE + DTILE, wave);
+        const bf16_t* Ab = A;
+        const bf16_t* Bb = B;
+        if constexpr (MULTI) {  // scalar selects: which pair K tile t belongs to
+            const bool s1 = t >= seg.t1, s2 = t >= seg.t2;
+            Ab = s2 ? seg.A2 : (s1 ? seg.A1 : A);
+            Bb = s2 ? seg.B2 : (s1 ? seg.B1 : B);
+            t -= s2 ? seg.t2 : (s1 ? seg.t1 : 0);
+        }
+        la.issue(Ab + (int64_t)t * astep, smem + stage * 2 * DTILE, wave);
+        lb.issue(Bb + (int64_t)t * bstep, smem + stage * 2 * DTILE + DTILE, wave);
     };
 
     issue_tile(0, 0);
@@ -398,6 +419,7 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
     // Pull the remaining kernel arguments into registers now: a scalar load still in flight inside the K loop shares the
     // counter of the LDS reads and would turn every counted wait on them into a full drain.
     asm volatile("" ::"s"(C), "s"(ldc), "s"(accumulate));
+    if constexpr (MULTI) asm volatile("" ::"s"(seg.A1), "s"(seg.B1), "s"(seg.A2), "s"(seg.B2), "s"(seg.t1), "s"(seg.t2));
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
     __syncthreads();
     read_b(smem, 0, 0);
@@ -589,5 +611,51 @@ extern "C" int ezl_gemm_bf16(const void* A, const void* B, void* C, int64_t M, i
     }
 #undef EZL_GEMM_CASE
     EZL_LAUNCH_CHECK("ezl_gemm_bf16");
+    return EZL_OK;
+}
+
+// C (=|+=) sum_i A[i] * B[i] over `count` operand pairs that share M, N and the leading dimensions; K[i] is the reduction
+// length of pair i.  The input gradient dx = sum_i dy_i W_i of linears that share their input is one such sum.  With up to
+// three pairs in the (a_kc = 1, b_kc = 0, bf16 output) form and every K[i] a positive multiple of 64 it is a single launch
+// that adds the products in fp32 and rounds once; otherwise the pairs go out as ezl_gemm_bf16 calls that accumulate into C.
+extern "C" int ezl_gemm_bf16_ksplit(int count, const void* const* A, const void* const* B, void* C, int64_t M, int64_t N,
+                                    const int64_t* K, int64_t lda, int64_t ldb, int64_t ldc, int a_kc, int b_kc, int out_dtype,
+                                    int accumulate, void* stream) {
+    EZL_REQUIRE(count >= 1 && A && B && K, EZL_EINVAL, "ezl_gemm_bf16_ksplit: bad count or null argument array");
+    bool one_launch = count <= 3 && a_kc == 1 && b_kc == 0 && out_dtype == 0 && M > 0 && N > 0;
+    int64_t ktot = 0;
+    for (int i = 0; i < count; ++i) {
+        EZL_REQUIRE(K[i] >= 0, EZL_EINVAL, "ezl_gemm_bf16_ksplit: negative size");
+        one_launch = one_launch && K[i] > 0 && K[i] % BK == 0;
+        ktot += K[i];
+    }
+    if (!one_launch || count == 1) {
+        for (int i = 0; i < count; ++i)
+            if (const int rc = ezl_gemm_bf16(A[i], B[i], C, M, N, K[i], lda, ldb, ldc, a_kc, b_kc, out_dtype, i == 0 ? accumulate : 1, stream))
+                return rc;
+        return EZL_OK;
+    }
+    EZL_REQUIRE(C, EZL_EINVAL, "ezl_gemm_bf16: null pointer");
+    for (int i = 0; i < count; ++i) {
+        EZL_REQUIRE(A[i] && B[i], EZL_EINVAL, "ezl_gemm_bf16: null pointer");
+        EZL_REQUIRE(ezl_aligned16(A[i]) && ezl_aligned16(B[i]) && lda % 8 == 0 && ldb % 8 == 0, EZL_EINVAL,
+                    "ezl_gemm_bf16: operands must be 16-byte aligned with leading dimensions that are multiples of 8");
+        EZL_REQUIRE(lda >= K[i] && M * lda < (1LL << 31) - 4096 && K[i] * ldb < (1LL << 31) - 4096, EZL_EUNSUPPORTED,
+                    "ezl_gemm_bf16: leading dimension too small or operand larger than 2^31 elements");
+    }
+    EZL_REQUIRE(N % 8 == 0 && ldb >= N && ldc >= N && M < (1LL << 31) && N < (1LL << 31) && ktot < (1LL << 31), EZL_EUNSUPPORTED,
+                "ezl_gemm_bf16: contiguous extent of B must be a multiple of 8");
+    const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    EZL_REQUIRE(tiles < (1LL << 31), EZL_EUNSUPPORTED, "ezl_gemm_bf16: too many tiles");
+    KSegments seg;
+    seg.A1 = (const bf16_t*)A[1]; seg.B1 = (const bf16_t*)B[1];
+    seg.t1 = (int)(K[0] / BK);
+    seg.A2 = count > 2 ? (const bf16_t*)A[2] : seg.A1; seg.B2 = count > 2 ? (const bf16_t*)B[2] : seg.B1;
+    seg.t2 = count > 2 ? (int)((K[0] + K[1]) / BK) : 0x7fffffff;
+    const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
+    hipLaunchKernelGGL((gemm_d2l_kernel<true, false, bf16_t, true>), dim3((unsigned)tiles), dim3(512), 0, (hipStream_t)stream,
+                       (const bf16_t*)A[0], (const bf16_t*)B[0], (bf16_t*)C, (int)M, (int)N, (int)ktot, lda, ldb, ldc, accumulate, tiles_m,
+                       tiles_n, seg);
+    EZL_LAUNCH_CHECK("ezl_gemm_bf16_ksplit");
     return EZL_OK;
 }

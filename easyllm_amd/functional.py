@@ -62,7 +62,8 @@ def linear(x, weight):
 
 class FanOutLinearFunction(torch.autograd.Function):
     """One input through several bias-free linears (q/k/v, or gate/up): y_i = x W_i^T.  The input gradient
-    sum_i dy_i W_i is accumulated inside the GEMM epilogue instead of by separate add kernels."""
+    sum_i dy_i W_i is one GEMM whose reduction runs over all (dy_i, W_i) pairs (fp32 sum, one rounding) instead of one
+    matmul per linear plus add kernels."""
 
     @staticmethod
     def forward(ctx, x, *weights):
@@ -76,15 +77,21 @@ class FanOutLinearFunction(torch.autograd.Function):
         x2d = x.reshape(-1, x.shape[-1])
         dx = None
         grads = []
-        for i, (dy, w) in enumerate(zip(dys, weights)):
+        dy2ds = []
+        for dy in dys:
             if dy is None:
-                grads.append(None)
+                dy2ds.append(None)
                 continue
             dy2d = dy.reshape(-1, dy.shape[-1])
-            if not dy2d.is_contiguous():
-                dy2d = dy2d.contiguous()
-            if ctx.needs_input_grad[0]:
-                dx = K.linear_dgrad(dy2d, w, out=dx, accumulate=dx is not None)
+            dy2ds.append(dy2d if dy2d.is_contiguous() else dy2d.contiguous())
+        if ctx.needs_input_grad[0]:
+            pairs = [(dy2d, w) for dy2d, w in zip(dy2ds, weights) if dy2d is not None]
+            if pairs:
+                dx = K.linear_dgrad_multi([a for a, _ in pairs], [b for _, b in pairs])
+        for i, (dy2d, w) in enumerate(zip(dy2ds, weights)):
+            if dy2d is None:
+                grads.append(None)
+                continue
             dw = None
             if ctx.needs_input_grad[1 + i]:
                 mg, acc = _main_grad_target(w)

@@ -218,6 +218,36 @@ def linear_dgrad(dy2d, w, out=None, accumulate=False):
     return gemm(dy2d, w, dy2d.shape[0], w.shape[1], w.shape[0], lda, ldb, True, False, out=out, accumulate=accumulate)
 
 
+def linear_dgrad_multi(dy2ds, ws, out=None, accumulate=False):
+    """dx[T, in] (=|+=) sum_i dy_i[T, out_i] @ w_i[out_i, in]: the input gradient of linears that share their input.
+    One launch when the dy_i share a row stride and the w_i theirs; otherwise one accumulating GEMM per pair."""
+    import ctypes
+    n = len(dy2ds)
+    _need(n == len(ws) and n >= 1, "linear_dgrad_multi: list lengths differ")
+    ldas = [_rows_ld(dy, "dy") for dy in dy2ds]
+    ldbs = [_rows_ld(w, "w") for w in ws]
+    T, n_in = dy2ds[0].shape[0], ws[0].shape[1]
+    for dy, w in zip(dy2ds, ws):
+        _need(dy.shape[1] == w.shape[0] and dy.shape[0] == T and w.shape[1] == n_in, "linear_dgrad: dimensions differ")
+    if len(set(ldas)) != 1 or len(set(ldbs)) != 1 or n > 3:
+        for i, (dy, w) in enumerate(zip(dy2ds, ws)):
+            out = linear_dgrad(dy, w, out=out, accumulate=accumulate or i > 0)
+        return out
+    if out is None:
+        out = torch.empty(T, n_in, dtype=BF16, device=dy2ds[0].device)
+    _need(out.is_cuda and out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (T, n_in) and out.dtype == BF16, "bad GEMM output")
+    if GEMM_TIMING is not None:
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+    _lib.call("ezl_gemm_bf16_ksplit", n, (ctypes.c_void_p * n)(*[_p(dy) for dy in dy2ds]), (ctypes.c_void_p * n)(*[_p(w) for w in ws]),
+              _p(out), T, n_in, (ctypes.c_int64 * n)(*[w.shape[0] for w in ws]), ldas[0], ldbs[0], out.stride(0), 1, 0, 0,
+              1 if accumulate else 0, _stream())
+    if GEMM_TIMING is not None:
+        end.record()
+        GEMM_TIMING.append((2.0 * T * n_in * sum(w.shape[0] for w in ws), start, end))
+    return out
+
+
 def linear_wgrad(dy2d, x2d, out=None, accumulate=False):
     """dw[out, in] (=|+=) dy[T, out]^T @ x[T, in]; `out` may be an fp32 main-grad buffer."""
     lda, ldb = _rows_ld(dy2d, "dy"), _rows_ld(x2d, "x")

@@ -179,6 +179,26 @@ def test_gemm_three_forms(K, gpu_device, T, n_in, n_out):
     close(mg, rdw, "gemm wgrad fp32 overwrite", rel=2e-3)
 
 
+@pytest.mark.parametrize("T,n_in,n_outs", [(512, 256, (256, 256, 256)), (300, 136, (128, 192)), (256, 256, (64, 1024, 64)),
+                                           (130, 64, (72, 64)), (256, 128, (128, 64))])
+def test_gemm_input_gradient_over_several_linears(K, gpu_device, T, n_in, n_outs):
+    """dx = sum_i dy_i W_i as one GEMM over all pairs (first three cases), and through the per-pair fallback (a reduction
+    length that is not a multiple of 64; dy_i with different row strides): against the fp32 sum, and `accumulate`."""
+    print("gemm dgrad multi", T, n_in, n_outs, flush=True)
+    ws = [rnd(n, n_in, seed=41 + i, scale=0.05) for i, n in enumerate(n_outs)]
+    dys = [rnd(T, n, seed=51 + i) for i, n in enumerate(n_outs)]
+    ref = sum(dy.float() @ w.float() for dy, w in zip(dys, ws))
+    wg, dyg = [w.to(gpu_device) for w in ws], [dy.to(gpu_device) for dy in dys]
+    dx = K.linear_dgrad_multi(dyg, wg)
+    close(dx, ref, "dgrad over several linears")
+    base = rnd(T, n_in, seed=61)
+    out = base.to(gpu_device).clone()
+    K.linear_dgrad_multi(dyg, wg, out=out, accumulate=True)
+    close(out, ref + base.float(), "dgrad over several linears, accumulate")
+    # the same call twice gives the same bits
+    assert torch.equal(dx, K.linear_dgrad_multi(dyg, wg))
+
+
 def test_gemm_forward_with_unaligned_output_width(K, gpu_device):
     """out features not a multiple of 4: the epilogue falls back from vector to element stores; K = 128 and 192 are the
     shortest reductions of the direct-to-LDS kernel (2 and 3 K tiles), K = 64 goes through the register-staged one."""
