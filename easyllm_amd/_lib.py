@@ -6,7 +6,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.environ.get("EZL_LIBRARY") or os.path.join(_HERE, "lib", "libezl.so")  # EZL_LIBRARY: another build of the same ABI
+LIB_PATH = os.path.join(_HERE, "lib", "libezl.so")
 
 _vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
 _i64p = ctypes.POINTER(ctypes.c_int64)
@@ -21,7 +21,7 @@ SIGNATURES = {
     "ezl_rope_table": [_vp, _vp, _vp, _i64, _i64, _f32, _vp],
     "ezl_rope_apply": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _vp],
     "ezl_embed_gather": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
-    "ezl_embed_scatter_add": [_vp, _vp, _vp, _i64, _i64, _i64, _vp],
+    "ezl_embed_scatter_add": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "ezl_transpose01": [_vp, _vp, _i64, _i64, _i64, _vp],
     "ezl_add": [_vp, _vp, _vp, _i64, _vp],
     "ezl_cast_bf16_to_f32": [_vp, _vp, _i64, _vp],
@@ -49,6 +49,7 @@ _SPECIAL = {
     "ezl_last_error": ([], ctypes.c_char_p),
     "ezl_rmsnorm_bwd_workspace_bytes": ([_i64, _i64], _i64),
     "ezl_bias_grad_workspace_bytes": ([_i64, _i64], _i64),
+    "ezl_embed_scatter_add_workspace_bytes": ([_i64, _i64], _i64),
     "ezl_sumsq_partials": ([], _i64),
     "ezl_location_idx_rows": ([_i64, _i64, _i64], _i64),
 }
@@ -96,6 +97,10 @@ def rmsnorm_bwd_workspace_bytes(rows, h):
 
 def bias_grad_workspace_bytes(rows, n):
     return load().ezl_bias_grad_workspace_bytes(rows, n)
+
+
+def embed_scatter_add_workspace_bytes(rows, vocab):
+    return load().ezl_embed_scatter_add_workspace_bytes(rows, vocab)
 
 
 def sumsq_partials():

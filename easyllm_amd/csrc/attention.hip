@@ -52,29 +52,78 @@ __device__ __forceinline__ int64_t tok_off(int n, int s_len, int64_t ss, int64_t
 // A document is cut at batch-row boundaries (the reference's collator never emits one that crosses a
 // row: it appends every row's length to that row's boundaries), so inside a document token i lives at
 // tok_off(doc_start) + i * seq_stride and no per-token division is needed.
+// The whole workgroup searches together (every thread must call this, before any other use of LDS): thread t counts the
+// blocks of documents t, t + blockDim.x, ..., a prefix sum over the workgroup locates the document that holds block
+// `bid`, and its thread publishes the answer -- ndocs / blockDim.x steps instead of a scalar walk over all documents.
+__device__ __forceinline__ int doc_bounds(const int* __restrict__ cu, int d, int s_len, int T, int& e) {
+    int a = cu ? cu[d] : d * s_len;
+    e = cu ? cu[d + 1] : (d + 1) * s_len;
+    a = a < 0 ? 0 : a;
+    e = e > T ? T : e;
+    return a;
+}
+
 __device__ __forceinline__ bool find_block(const int* __restrict__ cu, int ndocs, int s_len, int T, int bid, int blk_rows,
                                            int& doc_start, int& doc_len, int& blk) {
-    for (int d = 0; d < ndocs; ++d) {
-        int a = cu ? cu[d] : d * s_len;
-        int e = cu ? cu[d + 1] : (d + 1) * s_len;
-        a = a < 0 ? 0 : a;
-        e = e > T ? T : e;
-        while (a < e) {
-            const int row_end = (a / s_len + 1) * s_len;
-            const int e1 = e < row_end ? e : row_end;
-            const int len = e1 - a;
-            const int nb = (len + blk_rows - 1) / blk_rows;
-            if (bid < nb) {
-                doc_start = a;
-                doc_len = len;
-                blk = bid;
-                return true;
+    __shared__ int s_wave[16];
+    __shared__ int s_found[4];
+    const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63, wv = tid >> 6, nwaves = nthr >> 6;
+    if (tid == 0) s_found[0] = 0;
+    int base = 0;
+    for (int d0 = 0; d0 < ndocs; d0 += nthr) {
+        const int d = d0 + tid;
+        int nb = 0, a = 0, e = 0;
+        if (d < ndocs) {
+            a = doc_bounds(cu, d, s_len, T, e);
+            for (int x = a; x < e;) {  // one pass unless the document crosses a batch row
+                const int row_end = (x / s_len + 1) * s_len;
+                const int e1 = e < row_end ? e : row_end;
+                nb += (e1 - x + blk_rows - 1) / blk_rows;
+                x = e1;
             }
-            bid -= nb;
-            a = e1;
         }
+        int incl = nb;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += v;
+        }
+        __syncthreads();  // s_wave of the previous round has been read
+        if (lane == 63) s_wave[wv] = incl;
+        __syncthreads();
+        int before = 0, total = 0;
+        for (int i = 0; i < nwaves; ++i) {
+            const int v = s_wave[i];
+            before += i < wv ? v : 0;
+            total += v;
+        }
+        const int lo = base + before + incl - nb;  // first block id of this thread's document
+        if (nb > 0 && bid >= lo && bid < lo + nb) {
+            int rel = bid - lo;
+            for (int x = a; x < e;) {
+                const int row_end = (x / s_len + 1) * s_len;
+                const int e1 = e < row_end ? e : row_end;
+                const int n1 = (e1 - x + blk_rows - 1) / blk_rows;
+                if (rel < n1) {
+                    s_found[1] = x;
+                    s_found[2] = e1 - x;
+                    s_found[3] = rel;
+                    s_found[0] = 1;
+                    break;
+                }
+                rel -= n1;
+                x = e1;
+            }
+        }
+        base += total;
+        if (bid < base) break;  // uniform: the block lies in this round's documents
     }
-    return false;
+    __syncthreads();
+    if (!s_found[0]) return false;
+    doc_start = __builtin_amdgcn_readfirstlane(s_found[1]);
+    doc_len = __builtin_amdgcn_readfirstlane(s_found[2]);
+    blk = __builtin_amdgcn_readfirstlane(s_found[3]);
+    return true;
 }
 
 // The hardware deals consecutive workgroups (x fastest, then y) round-robin to the 8 XCDs, each with an L2 of its own.

@@ -284,6 +284,170 @@ __global__ __launch_bounds__(kCeBlock) void ce_fused_reg_kernel(const bf16_t* __
     }
 }
 
+// Fused loss + gradient for bf16 rows too long for the kernel above (a 152064-entry vocabulary): one 1024-thread block per
+// CU owns a row and keeps it RAW (bf16) on chip, so the logits are read from HBM exactly once and the gradient is written
+// once.  The first 9 x 1024 vectors of 8 logits live in LDS (144 KiB, thread t owns vector t of every 1024: private
+// slots, no barriers), the remaining NR x 1024 in registers.  exp is evaluated twice per element (sum pass, gradient
+// pass): fp32 copies would not fit.  While the gradient pass runs, each finished vector's slot is refilled with the
+// block's next row -- registers by a plain load, LDS slots by global_load_lds, which needs no registers at all -- so the
+// HBM pipe is busy under the vector ALU work.  Vectors past the row end hold -inf (exp = 0) and are never stored.
+constexpr int kWideBlock = 1024;
+constexpr int kWideWaves = kWideBlock / 64;
+constexpr int kWideLds = 9;  // vectors per thread kept in LDS
+
+typedef __attribute__((address_space(3))) void ce_lds_void;
+typedef __attribute__((address_space(1))) const void ce_gvoid;
+
+template <int NR, bool HAS_CUT>
+__global__ __launch_bounds__(kWideBlock) void ce_fused_wide_kernel(const bf16_t* __restrict__ logits, const int64_t* __restrict__ labels,
+                                                                   const float* __restrict__ weights, const float* __restrict__ count,
+                                                                   float* __restrict__ loss, bf16_t* __restrict__ grad, int64_t rows,
+                                                                   int V, int vend) {
+    __shared__ __attribute__((aligned(16))) bf16_t srow[kWideLds * kWideBlock * 8];
+    __shared__ float red[2][kWideWaves];
+    const int v8 = V >> 3;  // >= kWideLds * kWideBlock (checked by the host): every LDS vector lies inside the row
+    const float inv_n = 1.0f / count[0];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    bf16x8 raw[NR > 0 ? NR : 1];
+    auto fetch_reg = [&](const bf16_t* src, int j) {  // register vector j = row vector (kWideLds + j) * 1024 + tid
+        const int i = tid + (kWideLds + j) * kWideBlock;
+        if (i < v8) {
+            raw[j] = ld_bf16x8(src + (int64_t)i * 8);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) raw[j][k] = (bf16_t)(-INFINITY);
+        }
+    };
+    auto fetch_lds = [&](const bf16_t* src, int j) {  // one wave instruction fills the 64 slots of this wave in chunk j
+        __builtin_amdgcn_global_load_lds((ce_gvoid*)(src + (int64_t)(tid + j * kWideBlock) * 8),
+                                         (ce_lds_void*)(srow + (j * kWideBlock + wv * 64) * 8), 16, 0, 0);
+    };
+    auto lds_vec = [&](int j) { return *reinterpret_cast<const bf16x8*>(srow + (tid + j * kWideBlock) * 8); };
+
+    int64_t r = blockIdx.x;
+    if (r < rows) {
+        const bf16_t* src = logits + r * V;
+#pragma unroll
+        for (int j = 0; j < kWideLds; ++j) fetch_lds(src, j);
+#pragma unroll
+        for (int j = 0; j < NR; ++j) fetch_reg(src, j);
+    }
+    for (; r < rows; r += gridDim.x) {
+        const float w = weights[r];
+        bf16_t* grow = grad + r * V;
+        const int64_t rn = r + gridDim.x;
+        const bf16_t* next = logits + (rn < rows ? rn : r) * V;  // a block's last row re-reads itself (never used)
+        if (w == 0.f) {  // ignored position: exact zero gradient, contributes nothing to the loss
+            bf16x8 z;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) z[k] = (bf16_t)0.0f;
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this row's own loads into LDS have landed before they are replaced
+#pragma unroll
+            for (int j = 0; j < kWideLds; ++j) {
+                st_bf16x8(grow + (int64_t)(tid + j * kWideBlock) * 8, z);
+                fetch_lds(next, j);
+            }
+#pragma unroll
+            for (int j = 0; j < NR; ++j) {
+                const int i = tid + (kWideLds + j) * kWideBlock;
+                if (i < v8) st_bf16x8(grow + (int64_t)i * 8, z);
+                fetch_reg(next, j);
+            }
+            if (tid == 0) loss[r] = 0.f;
+            continue;
+        }
+        const int64_t t = labels[r];
+        const bool masked = t < 0 || t >= vend;
+        // the target logit straight from memory (the row is being read anyway): the passes below stay free of per-vector
+        // target tests, and the one-hot term is applied by a single-element fix-up after the gradient pass
+        const float xt = masked ? 0.f : (float)logits[r * V + t];
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the row is on chip (LDS part included)
+        asm volatile("" ::: "memory");           // ... and the compiler may not reuse LDS values read before this point
+        // ---- pass 1: row maximum over the columns below vend
+        float m = -INFINITY;
+        auto max_of = [&](const bf16x8 v, int i) {
+            float f[8];
+            unpack8(v, f);
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (!HAS_CUT || i * 8 + k < vend) m = fmaxf(m, f[k]);
+        };
+#pragma unroll
+        for (int j = 0; j < kWideLds; ++j) max_of(lds_vec(j), tid + j * kWideBlock);
+#pragma unroll
+        for (int j = 0; j < NR; ++j) max_of(raw[j], tid + (kWideLds + j) * kWideBlock);
+        m = wave_max(m);
+        __syncthreads();  // red is free again (read by every thread at the end of the previous row)
+        if (lane == 0) red[0][wv] = m;
+        __syncthreads();
+        m = red[0][0];
+#pragma unroll
+        for (int i = 1; i < kWideWaves; ++i) m = fmaxf(m, red[0][i]);
+        const float mb = m * kLog2e;
+        // ---- pass 2: sum of exp(x - max) over the columns below vend
+        float ssum = 0.f;
+        auto sum_of = [&](const bf16x8 v, int i) {
+            float f[8];
+            unpack8(v, f);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const float e = __builtin_amdgcn_exp2f(f[k] * kLog2e - mb);
+                if (!HAS_CUT || i * 8 + k < vend) ssum += e;
+            }
+        };
+#pragma unroll
+        for (int j = 0; j < kWideLds; ++j) sum_of(lds_vec(j), tid + j * kWideBlock);
+#pragma unroll
+        for (int j = 0; j < NR; ++j) {
+            asm volatile("" : "+v"(raw[j]));  // opaque: the fp32 copies of pass 1 must not be kept alive
+            sum_of(raw[j], tid + (kWideLds + j) * kWideBlock);
+        }
+        ssum = wave_sum(ssum);
+        if (lane == 0) red[1][wv] = ssum;
+        __syncthreads();
+        ssum = 0.f;
+#pragma unroll
+        for (int i = 0; i < kWideWaves; ++i) ssum += red[1][i];
+        const float lse = m + logf(ssum);
+        if (tid == 0) loss[r] = masked ? logf(ssum) : (lse - xt);
+        const float scale = w * inv_n;
+        const float ps = scale / ssum;  // exp(x - lse) * scale = exp(x - max) * scale / sum
+        // ---- pass 3: gradient; the exponentials are evaluated again on purpose.  The copy of `mb` is opaque to the
+        // compiler, which would otherwise recognise the expression of pass 2, keep all of that pass's results alive across
+        // the block reduction and spill them.
+        float mb2 = mb;
+        asm volatile("" : "+v"(mb2));
+        auto grad_of = [&](const bf16x8 v) {
+            float g[8];
+            unpack8(v, g);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) g[k] = __builtin_amdgcn_exp2f(g[k] * kLog2e - mb2) * ps;
+            return pack8(g);
+        };
+#pragma unroll
+        for (int j = 0; j < kWideLds; ++j) {
+            const int i = tid + j * kWideBlock;
+            st_bf16x8(grow + (int64_t)i * 8, grad_of(lds_vec(j)));
+            // the LDS read above has returned (its value was used): the slot may be refilled with the next row
+            fetch_lds(next, j);
+        }
+#pragma unroll
+        for (int j = 0; j < NR; ++j) {
+            const int i = tid + (kWideLds + j) * kWideBlock;
+            asm volatile("" : "+v"(raw[j]));
+            const bf16x8 gv = grad_of(raw[j]);
+            if (i < v8) st_bf16x8(grow + (int64_t)i * 8, gv);
+            fetch_reg(next, j);  // this vector's registers are free: start the next row's fetch behind the store
+        }
+        // one-hot term: the thread that stored the vector holding the target column rewrites that one element (stores of
+        // one thread to one address keep their order)
+        if (!masked && tid == (int)((t >> 3) & (kWideBlock - 1)))
+            grow[t] = (bf16_t)(__builtin_amdgcn_exp2f(xt * kLog2e - mb2) * ps - scale);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // no LDS write of this block may still be in flight when it ends
+}
+
 // weights[i] = mask[i] * (labels[i] != ignore_index); count[0] = sum(weights) -- one block, fixed order
 __global__ __launch_bounds__(1024) void ce_prepare_kernel(const int64_t* __restrict__ labels, const void* __restrict__ mask,
                                                           int mask_dtype, int64_t ignore_index, float* __restrict__ weights,
@@ -421,7 +585,24 @@ extern "C" int ezl_ce_fused(const void* logits, const void* labels, const void* 
         if (V <= kCeBlock * 8 * 2) { if (cut) LAUNCH((ce_fused_reg_kernel<2, true>), bf16_t, 0); else LAUNCH((ce_fused_reg_kernel<2, false>), bf16_t, 0); }
         else if (V <= kCeBlock * 8 * 4) { if (cut) LAUNCH((ce_fused_reg_kernel<4, true>), bf16_t, 0); else LAUNCH((ce_fused_reg_kernel<4, false>), bf16_t, 0); }
         else if (V <= kCeBlock * 8 * 8) { if (cut) LAUNCH((ce_fused_reg_kernel<8, true>), bf16_t, 0); else LAUNCH((ce_fused_reg_kernel<8, false>), bf16_t, 0); }
-        else LAUNCH((ce_fused_kernel<bf16_t, false>), bf16_t, 0);
+        else if (V >= kWideBlock * 8 * kWideLds && V <= kWideBlock * 8 * (kWideLds + 13)) {
+            // one block per CU (1024 threads, 144 KiB of LDS); every block walks rows blockIdx.x, + gridDim.x, ...
+            const unsigned g = (unsigned)(rows < 256 ? rows : 256);
+#define LAUNCH_WIDE(NR)                                                                                                       \
+    do {                                                                                                                      \
+        if (cut) hipLaunchKernelGGL((ce_fused_wide_kernel<NR, true>), dim3(g), dim3(kWideBlock), 0, st, (const bf16_t*)logits, \
+                                    (const int64_t*)labels, (const float*)weights, (const float*)count, (float*)loss_rows,    \
+                                    (bf16_t*)grad, rows, V, vend);                                                            \
+        else hipLaunchKernelGGL((ce_fused_wide_kernel<NR, false>), dim3(g), dim3(kWideBlock), 0, st, (const bf16_t*)logits,    \
+                                (const int64_t*)labels, (const float*)weights, (const float*)count, (float*)loss_rows,        \
+                                (bf16_t*)grad, rows, V, vend);                                                                \
+    } while (0)
+            if (V <= kWideBlock * 8 * (kWideLds + 4)) LAUNCH_WIDE(4);
+            else if (V <= kWideBlock * 8 * (kWideLds + 7)) LAUNCH_WIDE(7);
+            else if (V <= kWideBlock * 8 * (kWideLds + 10)) LAUNCH_WIDE(10);
+            else LAUNCH_WIDE(13);
+#undef LAUNCH_WIDE
+        } else LAUNCH((ce_fused_kernel<bf16_t, false>), bf16_t, 0);
     } else {
         if (in_lds) LAUNCH((ce_fused_kernel<float, true>), float, row_bytes); else LAUNCH((ce_fused_kernel<float, false>), float, 0);
     }

@@ -133,54 +133,134 @@ __global__ __launch_bounds__(kBlock) void embed_gather_kernel(const int64_t* __r
     }
 }
 
-// dW[id, :] += sum of dY[r, :] over all rows r with ids[r] == id, without atomics and in a fixed order:
-// the block of the FIRST row holding an id owns that id; it scans the later rows 256 at a time and adds the
-// (rare) duplicates in increasing row order, then does one read-modify-write of the fp32 row.
+// dW[id, :] += sum of dY[r, :] over all rows r with ids[r] == id, in increasing row order (bit-reproducible), in time
+// linear in the number of rows.  The rows are bucketed by id through four int32 tables in the workspace:
+//   cnt[V]   rows per id                      first[V]  smallest row holding the id (its block does the sum)
+//   off[V]   exclusive prefix sum of cnt      bucket[T] rows grouped by id (order inside a group: as the atomics fell)
+// The owner block of an id sorts that id's bucket by row number before summing, so the order the atomics produced never
+// reaches the result.
+constexpr int kScanThreads = 1024;
+constexpr int kBucketLds = 1024;  // buckets up to this size are sorted in LDS; longer ones by repeated selection
+
+__global__ __launch_bounds__(kBlock) void embed_tables_init_kernel(int* __restrict__ cnt, int* __restrict__ first,
+                                                                   int* __restrict__ fill, int64_t V) {
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < V; i += (int64_t)gridDim.x * kBlock) {
+        cnt[i] = 0;
+        fill[i] = 0;
+        first[i] = 0x7fffffff;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void embed_count_kernel(const int64_t* __restrict__ ids, int* __restrict__ cnt,
+                                                             int* __restrict__ first, int64_t rows, int64_t V) {
+    for (int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x; r < rows; r += (int64_t)gridDim.x * kBlock) {
+        const int64_t id = ids[r];
+        if (id < 0 || id >= V) continue;
+        atomicAdd(cnt + id, 1);
+        atomicMin(first + id, (int)r);
+    }
+}
+
+// off = exclusive prefix sum of cnt over V entries: one block, each thread a contiguous run
+__global__ __launch_bounds__(kScanThreads) void embed_scan_kernel(const int* __restrict__ cnt, int* __restrict__ off, int64_t V) {
+    __shared__ int part[kScanThreads];
+    const int64_t per = (V + kScanThreads - 1) / kScanThreads;
+    const int64_t lo = (int64_t)threadIdx.x * per, hi = lo + per < V ? lo + per : V;
+    int sum = 0;
+    for (int64_t i = lo; i < hi; ++i) sum += cnt[i];
+    part[threadIdx.x] = sum;
+    __syncthreads();
+    for (int d = 1; d < kScanThreads; d <<= 1) {  // inclusive scan of the per-thread sums
+        const int v = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+        __syncthreads();
+        part[threadIdx.x] += v;
+        __syncthreads();
+    }
+    int run = part[threadIdx.x] - sum;
+    for (int64_t i = lo; i < hi; ++i) {
+        off[i] = run;
+        run += cnt[i];
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void embed_bucket_kernel(const int64_t* __restrict__ ids, const int* __restrict__ off,
+                                                              int* __restrict__ fill, int* __restrict__ bucket, int64_t rows,
+                                                              int64_t V) {
+    for (int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x; r < rows; r += (int64_t)gridDim.x * kBlock) {
+        const int64_t id = ids[r];
+        if (id < 0 || id >= V) continue;
+        bucket[off[id] + atomicAdd(fill + id, 1)] = (int)r;
+    }
+}
+
 template <int MAXC>
-__global__ __launch_bounds__(kBlock) void embed_scatter_owner_kernel(const int64_t* __restrict__ ids, const bf16_t* __restrict__ dY,
-                                                                     float* __restrict__ dW, int64_t rows, int h, int64_t V) {
-    __shared__ unsigned long long bits[kBlock / 64];
+__global__ __launch_bounds__(kBlock) void embed_scatter_bucket_kernel(const int64_t* __restrict__ ids, const bf16_t* __restrict__ dY,
+                                                                      float* __restrict__ dW, const int* __restrict__ cnt,
+                                                                      const int* __restrict__ first, const int* __restrict__ off,
+                                                                      const int* __restrict__ bucket, int64_t rows, int h,
+                                                                      int64_t V) {
+    __shared__ int raw[kBucketLds];
+    __shared__ int sorted[kBucketLds];
+    __shared__ int wmin[kBlock / 64];
     const int h8 = h >> 3;
     for (int64_t t = blockIdx.x; t < rows; t += gridDim.x) {
         const int64_t id = ids[t];
         if (id < 0 || id >= V) continue;
-        int earlier = 0;
-        for (int64_t j = threadIdx.x; j < t; j += kBlock) earlier |= (ids[j] == id);
-        if (__syncthreads_or(earlier)) continue;  // an earlier row owns this id
+        if (first[id] != (int)t) continue;  // the block of the smallest row of an id owns it (uniform over the block)
+        const int n = cnt[id];
+        const int* mine = bucket + off[id];
         float acc[MAXC][8];
 #pragma unroll
-        for (int c = 0; c < MAXC; ++c) {
-            const int col = (c * kBlock + threadIdx.x);
+        for (int c = 0; c < MAXC; ++c)
 #pragma unroll
             for (int k = 0; k < 8; ++k) acc[c][k] = 0.f;
-            if (col < h8) unpack8(ld_bf16x8(dY + t * h + col * 8), acc[c]);
-        }
-        for (int64_t base = t + 1; base < rows; base += kBlock) {
-            const int64_t j = base + threadIdx.x;
-            const int match = (j < rows) && (ids[j] == id);
-            if (__syncthreads_or(match)) {
-                const unsigned long long b = __ballot(match);
-                if ((threadIdx.x & 63) == 0) bits[threadIdx.x >> 6] = b;
-                __syncthreads();
-                for (int wv = 0; wv < kBlock / 64; ++wv) {
-                    unsigned long long m = bits[wv];
-                    while (m) {
-                        const int l = __builtin_ctzll(m);
-                        m &= m - 1;
-                        const int64_t jj = base + wv * 64 + l;
+        auto add_row = [&](int64_t jj) {
 #pragma unroll
-                        for (int c = 0; c < MAXC; ++c) {
-                            const int col = (c * kBlock + threadIdx.x);
-                            if (col < h8) {
-                                float g[8];
-                                unpack8(ld_bf16x8(dY + jj * h + col * 8), g);
+            for (int c = 0; c < MAXC; ++c) {
+                const int col = (c * kBlock + threadIdx.x);
+                if (col < h8) {
+                    float g[8];
+                    unpack8(ld_bf16x8(dY + jj * h + col * 8), g);
 #pragma unroll
-                                for (int k = 0; k < 8; ++k) acc[c][k] += g[k];
-                            }
-                        }
-                    }
+                    for (int k = 0; k < 8; ++k) acc[c][k] += g[k];
+                }
+            }
+        };
+        if (n == 1) {
+            add_row(t);
+        } else if (n <= kBucketLds) {
+            __syncthreads();  // the previous id's LDS use is over
+            for (int i = threadIdx.x; i < n; i += kBlock) raw[i] = mine[i];
+            __syncthreads();
+            for (int i = threadIdx.x; i < n; i += kBlock) {  // rows are distinct: rank = number of smaller rows
+                const int v = raw[i];
+                int rank = 0;
+                for (int j = 0; j < n; ++j) rank += raw[j] < v;
+                sorted[rank] = v;
+            }
+            __syncthreads();
+            for (int i = 0; i < n; ++i) add_row(sorted[i]);
+        } else {
+            int prev = -1;
+            for (int i = 0; i < n; ++i) {  // next row = the smallest bucket entry above the previous one
+                int m = 0x7fffffff;
+                for (int j = threadIdx.x; j < n; j += kBlock) {
+                    const int v = mine[j];
+                    if (v > prev && v < m) m = v;
+                }
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) {
+                    const int other = __shfl_xor(m, o, 64);
+                    m = other < m ? other : m;
                 }
                 __syncthreads();
+                if ((threadIdx.x & 63) == 0) wmin[threadIdx.x >> 6] = m;
+                __syncthreads();
+                m = wmin[0];
+#pragma unroll
+                for (int wv = 1; wv < kBlock / 64; ++wv) m = wmin[wv] < m ? wmin[wv] : m;
+                add_row(m);
+                prev = m;
             }
         }
 #pragma unroll
@@ -343,24 +423,46 @@ extern "C" int ezl_embed_gather(const void* ids, const void* weight, void* out, 
     return EZL_OK;
 }
 
-extern "C" int ezl_embed_scatter_add(const void* ids, const void* dy, void* dweight_f32, int64_t rows, int64_t h,
-                                     int64_t vocab, void* stream) {
+extern "C" int64_t ezl_embed_scatter_add_workspace_bytes(int64_t rows, int64_t vocab) {
+    if (rows < 0 || vocab <= 0) return -1;
+    return (4 * vocab + rows) * (int64_t)sizeof(int);
+}
+
+extern "C" int ezl_embed_scatter_add(const void* ids, const void* dy, void* dweight_f32, void* workspace, int64_t workspace_bytes,
+                                     int64_t rows, int64_t h, int64_t vocab, void* stream) {
     EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h < (1LL << 31) && vocab > 0, EZL_EUNSUPPORTED,
                 "ezl_embed_scatter_add: h must be a multiple of 8");
     EZL_REQUIRE((rows == 0 || (ids && dy && dweight_f32)) && ezl_aligned16(dy), EZL_EINVAL,
                 "ezl_embed_scatter_add: null or misaligned pointer");
     if (rows == 0) return EZL_OK;
     EZL_REQUIRE(h <= 8192 * 2, EZL_EUNSUPPORTED, "ezl_embed_scatter_add: h must be <= 16384");
+    EZL_REQUIRE(rows < (1LL << 31) && vocab < (1LL << 31), EZL_EUNSUPPORTED, "ezl_embed_scatter_add: more than 2^31 rows or ids");
     EZL_REQUIRE(((uintptr_t)dweight_f32 & 15) == 0, EZL_EINVAL, "ezl_embed_scatter_add: dweight must be 16-byte aligned");
+    EZL_REQUIRE(workspace && ((uintptr_t)workspace & 3) == 0 && workspace_bytes >= ezl_embed_scatter_add_workspace_bytes(rows, vocab),
+                EZL_EINVAL, "ezl_embed_scatter_add: workspace missing or smaller than ezl_embed_scatter_add_workspace_bytes()");
+    int* cnt = (int*)workspace;
+    int* first = cnt + vocab;
+    int* off = first + vocab;
+    int* fill = off + vocab;
+    int* bucket = fill + vocab;
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(embed_tables_init_kernel, dim3(grid_for(vocab, kBlock, 1024)), dim3(kBlock), 0, st, cnt, first, fill, vocab);
+    hipLaunchKernelGGL(embed_count_kernel, dim3(grid_for(rows, kBlock, 1024)), dim3(kBlock), 0, st, (const int64_t*)ids, cnt, first,
+                       rows, vocab);
+    hipLaunchKernelGGL(embed_scan_kernel, dim3(1), dim3(kScanThreads), 0, st, cnt, off, vocab);
+    hipLaunchKernelGGL(embed_bucket_kernel, dim3(grid_for(rows, kBlock, 1024)), dim3(kBlock), 0, st, (const int64_t*)ids, off, fill,
+                       bucket, rows, vocab);
+    EZL_LAUNCH_CHECK("ezl_embed_scatter_add(tables)");
+    const dim3 grid(grid_for(rows, 1));
     if (h <= 8 * kBlock * 2)
-        hipLaunchKernelGGL((embed_scatter_owner_kernel<2>), dim3(grid_for(rows, 1)), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const int64_t*)ids, (const bf16_t*)dy, (float*)dweight_f32, rows, (int)h, vocab);
+        hipLaunchKernelGGL((embed_scatter_bucket_kernel<2>), grid, dim3(kBlock), 0, st, (const int64_t*)ids, (const bf16_t*)dy,
+                           (float*)dweight_f32, cnt, first, off, bucket, rows, (int)h, vocab);
     else if (h <= 8 * kBlock * 4)
-        hipLaunchKernelGGL((embed_scatter_owner_kernel<4>), dim3(grid_for(rows, 1)), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const int64_t*)ids, (const bf16_t*)dy, (float*)dweight_f32, rows, (int)h, vocab);
+        hipLaunchKernelGGL((embed_scatter_bucket_kernel<4>), grid, dim3(kBlock), 0, st, (const int64_t*)ids, (const bf16_t*)dy,
+                           (float*)dweight_f32, cnt, first, off, bucket, rows, (int)h, vocab);
     else
-        hipLaunchKernelGGL((embed_scatter_owner_kernel<8>), dim3(grid_for(rows, 1)), dim3(kBlock), 0, (hipStream_t)stream,
-                           (const int64_t*)ids, (const bf16_t*)dy, (float*)dweight_f32, rows, (int)h, vocab);
+        hipLaunchKernelGGL((embed_scatter_bucket_kernel<8>), grid, dim3(kBlock), 0, st, (const int64_t*)ids, (const bf16_t*)dy,
+                           (float*)dweight_f32, cnt, first, off, bucket, rows, (int)h, vocab);
     EZL_LAUNCH_CHECK("ezl_embed_scatter_add");
     return EZL_OK;
 }

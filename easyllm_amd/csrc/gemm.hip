@@ -141,8 +141,11 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_staged_kernel(con
 
     Stager<A_KC, NT, KTAIL> sa;
     Stager<B_KC, NT, KTAIL> sb;
-    sa.init(tid, m0, M, lda);
-    sb.init(tid, n0, N, ldb);
+    // per-thread offsets are 32-bit and relative to the block's first row / column: operands of any size are addressable
+    A += A_KC ? (int64_t)m0 * lda : (int64_t)m0;
+    B += B_KC ? (int64_t)n0 * ldb : (int64_t)n0;
+    sa.init(tid, 0, M - m0, lda);
+    sb.init(tid, 0, N - n0, ldb);
     constexpr int NCH = 2048 / NT;
     bf16x8 ra[NCH], rb[NCH];
 
@@ -367,8 +370,12 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
 
     Loader<A_KC, NW> la;
     Loader<B_KC, NW> lb;
-    la.init(lane, wave, m0, M, lda);
-    lb.init(lane, wave, n0, N, ldb);
+    // per-lane offsets are 32-bit and relative to the block's first row / column (a scalar 64-bit advance of the operand
+    // base), so operands of more than 2^31 elements are addressable
+    const int64_t a_blk = A_KC ? (int64_t)m0 * lda : (int64_t)m0;
+    const int64_t b_blk = B_KC ? (int64_t)n0 * ldb : (int64_t)n0;
+    la.init(lane, wave, 0, M - m0, lda);
+    lb.init(lane, wave, 0, N - n0, ldb);
 
     f32x4 acc[8][4];
 #pragma unroll
@@ -410,8 +417,8 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
             Bb = s2 ? seg.B2 : (s1 ? seg.B1 : B);
             t -= s2 ? seg.t2 : (s1 ? seg.t1 : 0);
         }
-        la.issue(Ab + (int64_t)t * astep, smem + stage * 2 * DTILE, wave);
-        lb.issue(Bb + (int64_t)t * bstep, smem + stage * 2 * DTILE + DTILE, wave);
+        la.issue(Ab + a_blk + (int64_t)t * astep, smem + stage * 2 * DTILE, wave);
+        lb.issue(Bb + b_blk + (int64_t)t * bstep, smem + stage * 2 * DTILE + DTILE, wave);
     };
 
     issue_tile(0, 0);
@@ -591,9 +598,9 @@ extern "C" int ezl_gemm_bf16(const void* A, const void* B, void* C, int64_t M, i
     EZL_REQUIRE(a_kc ? (K % 8 == 0) : (M % 8 == 0), EZL_EUNSUPPORTED, "ezl_gemm_bf16: contiguous extent of A must be a multiple of 8");
     EZL_REQUIRE(b_kc ? (K % 8 == 0) : (N % 8 == 0), EZL_EUNSUPPORTED, "ezl_gemm_bf16: contiguous extent of B must be a multiple of 8");
     EZL_REQUIRE(lda >= (a_kc ? K : M) && ldb >= (b_kc ? K : N) && ldc >= N, EZL_EINVAL, "ezl_gemm_bf16: leading dimension too small");
-    const int64_t a_rows = a_kc ? M : K, b_rows = b_kc ? N : K;
-    EZL_REQUIRE(a_rows * lda < (1LL << 31) - 4096 && b_rows * ldb < (1LL << 31) - 4096 && M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31),
-                EZL_EUNSUPPORTED, "ezl_gemm_bf16: operand larger than 2^31 elements");
+    // 32-bit byte offsets inside one 256-row (or 64-k-row) tile; the tile bases advance in 64 bits
+    EZL_REQUIRE(lda < (1LL << 22) && ldb < (1LL << 22) && M < (1LL << 31) && N < (1LL << 31) && K < (1LL << 31), EZL_EUNSUPPORTED,
+                "ezl_gemm_bf16: a dimension of 2^31 or more, or a leading dimension of 2^22 or more");
     const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     EZL_REQUIRE(tiles < (1LL << 31), EZL_EUNSUPPORTED, "ezl_gemm_bf16: too many tiles");
     hipStream_t st = (hipStream_t)stream;
@@ -640,8 +647,8 @@ extern "C" int ezl_gemm_bf16_ksplit(int count, const void* const* A, const void*
         EZL_REQUIRE(A[i] && B[i], EZL_EINVAL, "ezl_gemm_bf16: null pointer");
         EZL_REQUIRE(ezl_aligned16(A[i]) && ezl_aligned16(B[i]) && lda % 8 == 0 && ldb % 8 == 0, EZL_EINVAL,
                     "ezl_gemm_bf16: operands must be 16-byte aligned with leading dimensions that are multiples of 8");
-        EZL_REQUIRE(lda >= K[i] && M * lda < (1LL << 31) - 4096 && K[i] * ldb < (1LL << 31) - 4096, EZL_EUNSUPPORTED,
-                    "ezl_gemm_bf16: leading dimension too small or operand larger than 2^31 elements");
+        EZL_REQUIRE(lda >= K[i] && lda < (1LL << 22) && ldb < (1LL << 22), EZL_EUNSUPPORTED,
+                    "ezl_gemm_bf16: leading dimension too small, or 2^22 or more");
     }
     EZL_REQUIRE(N % 8 == 0 && ldb >= N && ldc >= N && M < (1LL << 31) && N < (1LL << 31) && ktot < (1LL << 31), EZL_EUNSUPPORTED,
                 "ezl_gemm_bf16: contiguous extent of B must be a multiple of 8");

@@ -1,8 +1,9 @@
 """Integer producers of the packed-sequence inputs and the batch tuple layout the model consumes.
 
-Reference: `get_cu_seqlens` / `get_position_ids` (llm/data/nlp_transforms.py:40-55), the per-batch
-flattening of cu_seqlens in `BatchAlignCollector._pad_func` (llm/data/nlp_dataloader.py:172-187) and
-the tuple layouts of `json_batch_pipe` / `flash_batch_pipe` (llm/data/nlp_batch_fn.py:131-205).
+Reference: `get_cu_seqlens` / `get_position_ids` (llm/data/nlp_transforms.py:40-55), the collator
+`BatchAlignCollector` (llm/data/nlp_dataloader.py:110-187: next-token shift, padding, per-batch
+flattening of cu_seqlens) and the tuple layouts of `json_batch_pipe` / `flash_batch_pipe`
+(llm/data/nlp_batch_fn.py:131-205).
 Host-side numpy/torch integer code; nothing here is in the timed region.
 """
 import numpy as np
@@ -36,6 +37,43 @@ def flatten_cu_seqlens(cu_list, max_seq_length):
         c = torch.clamp(torch.as_tensor(cu, dtype=torch.int64), max=max_seq_length) + bidx * max_seq_length
         parts.append(c if bidx == 0 else c[1:])
     return torch.cat(parts)
+
+
+def _pad_with_alignment(items, padding_value, max_seq_length, alignment, offset_label, is_label):
+    """nlp_dataloader.py:147-170: rows padded to the batch's longest item (rounded up to `alignment`, capped at
+    max_seq_length); with offset_label the inputs drop their last token and the labels their first (next-token shift)."""
+    new_size = -(-max(len(it) for it in items) // alignment) * alignment
+    rows = []
+    for it in items:
+        row = torch.full((min(max_seq_length, new_size),), padding_value, dtype=torch.int64)
+        o_size = it.size(0) - 1
+        if offset_label:
+            row[:o_size] = it[1:] if is_label else it[:-1]
+        else:
+            row[:o_size + 1] = it[:max_seq_length]
+        rows.append(row)
+    return torch.stack(rows)
+
+
+def batch_align_collate(instances, pad_token_id, max_seq_length, alignment=1, ignore_idx=IGNORE_INDEX, offset_label=True,
+                        pretrain=False):
+    """`BatchAlignCollector.__call__` (nlp_dataloader.py:131-145): dataset items -> dict of batch tensors.  With
+    `pretrain`, items carry `cu_seqlens` / `position_ids` (packed samples) and the batch gets the flattened boundaries."""
+    input_ids = _pad_with_alignment([i["input_ids"] for i in instances], pad_token_id, max_seq_length, alignment, offset_label, False)
+    labels = _pad_with_alignment([i["labels"] for i in instances], ignore_idx, max_seq_length, alignment, offset_label, True)
+    batch = dict(input_ids=input_ids, labels=labels, attention_mask=input_ids.ne(pad_token_id))
+    if pretrain:
+        batch["position_ids"] = _pad_with_alignment([i["position_ids"] for i in instances], 0, max_seq_length, alignment,
+                                                    offset_label, False)
+        batch["cu_seqlens"] = flatten_cu_seqlens([i["cu_seqlens"] for i in instances], max_seq_length)
+    return batch
+
+
+def flash_batch_from(batch, pad_token_id, pretrain=False):
+    """`FlashBatchFunction.__call__` (nlp_batch_fn.py:181-205) on a collated batch dict."""
+    if pretrain:
+        return flash_batch(batch["input_ids"].long(), batch["labels"].long(), pad_token_id, batch["cu_seqlens"], batch["position_ids"])
+    return flash_batch(batch["input_ids"].long(), batch["labels"].long(), pad_token_id)
 
 
 def flash_batch(tokens, labels, pad_token_id, cu_seqlens=None, position_ids=None):

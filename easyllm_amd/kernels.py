@@ -134,7 +134,9 @@ def embed_scatter_add(ids, dy, dweight_f32):
     _bf16c(dy, "dy")
     V, h = dweight_f32.shape
     _need(dweight_f32.dtype == torch.float32 and dweight_f32.is_contiguous() and dy.shape[-1] == h, "bad dweight")
-    _lib.call("ezl_embed_scatter_add", _p(ids), _p(dy), _p(dweight_f32), ids.numel(), h, V, _stream())
+    ws_bytes = _lib.embed_scatter_add_workspace_bytes(ids.numel(), V)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dy.device)
+    _lib.call("ezl_embed_scatter_add", _p(ids), _p(dy), _p(dweight_f32), _p(ws), ws_bytes, ids.numel(), h, V, _stream())
 
 
 # ------------------------------------------------------------------------------------- plumbing
@@ -194,7 +196,27 @@ def gemm(A, B, M, N, K, lda, ldb, a_kc, b_kc, out=None, out_dtype=BF16, accumula
     return _gemm(A, B, M, N, K, lda, ldb, a_kc, b_kc, out, out_dtype, accumulate)
 
 
+def _span(t):
+    """Elements from the tensor's first element to one past its last (views of a wider matrix included)."""
+    if t.numel() == 0:
+        return 0
+    return 1 + sum((n - 1) * st for n, st in zip(t.shape, t.stride()))
+
+
+def _extent_ok(t, rows, cols, ld):
+    """True when a [rows x cols] operand with leading dimension ld lies inside tensor t."""
+    if rows == 0 or cols == 0:
+        return True
+    return ld >= cols and _span(t) >= (rows - 1) * ld + cols
+
+
 def _gemm(A, B, M, N, K, lda, ldb, a_kc, b_kc, out, out_dtype, accumulate):
+    _need(not (accumulate and out is None), "GEMM: accumulate needs the buffer to add to (out=...)")
+    for t, name in ((A, "A"), (B, "B")):
+        _need(t.is_cuda and t.dtype == BF16 and t.stride(-1) == 1, "GEMM operand %s must be a bf16 GPU tensor with unit inner stride" % name)
+    # A is M x K stored [m][k] (a_kc) or [k][m]; B is N x K stored [n][k] (b_kc) or [k][n]
+    _need(_extent_ok(A, M, K, lda) if a_kc else _extent_ok(A, K, M, lda), "GEMM: A is smaller than M x K with this leading dimension")
+    _need(_extent_ok(B, N, K, ldb) if b_kc else _extent_ok(B, K, N, ldb), "GEMM: B is smaller than N x K with this leading dimension")
     if out is None:
         out = torch.empty(M, N, dtype=out_dtype, device=A.device)
     _need(out.is_cuda and out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (M, N), "bad GEMM output")
@@ -224,6 +246,7 @@ def linear_dgrad_multi(dy2ds, ws, out=None, accumulate=False):
     import ctypes
     n = len(dy2ds)
     _need(n == len(ws) and n >= 1, "linear_dgrad_multi: list lengths differ")
+    _need(not (accumulate and out is None), "linear_dgrad_multi: accumulate needs the buffer to add to (out=...)")
     ldas = [_rows_ld(dy, "dy") for dy in dy2ds]
     ldbs = [_rows_ld(w, "w") for w in ws]
     T, n_in = dy2ds[0].shape[0], ws[0].shape[1]

@@ -4,14 +4,19 @@ Counterpart of llm/data/data_utils.py:106-260 (`MMapIndex`, `MMapIndexedDatasetB
 version 1, dtype code, sizes int32, byte pointers int64, document index int64) and of `MMapIndexJsonDataset`
 (llm/data/nlp_dataset.py:322-646) from the point where the token cache exists: the three index maps (document order
 per epoch, sample locations, sample shuffle), sample extraction, and `cu_seqlens` / `position_ids` emission for the
-packed attention path.  Building the cache from json through a tokenizer + transform pipeline is not part of this file;
-`MMapIndexedDatasetBuilder` writes caches from token arrays.
+packed attention path.  `build_data_cache` writes the cache from line-json files (data_utils.py:268-385): every line
+goes through an `encode` callable -- the reference's tokenizer + transform pipeline, which is not part of this build, or
+by default a reader of already tokenised lines `{"input_ids": [...]}` -- and becomes one document of the cache.
 
 The sample-location table comes from the native builder (`ezl_build_location_idx`), which replaces the reference's
 pybind11 helper; there is no python fallback for it.
 """
+import json
 import os
+import shutil
 import struct
+import tempfile
+from multiprocessing import Pool
 
 import numpy as np
 import torch
@@ -104,9 +109,95 @@ class MMapIndexedDatasetBuilder:
     def end_document(self):
         self._doc_idx.append(len(self._sizes))
 
+    def merge_file_(self, another_prefix):
+        """Appends the cache `<another_prefix>.idx/.bin` (data_utils.py:234-248)."""
+        index = MMapIndex(index_file_path(another_prefix))
+        assert index.dtype == self._dtype
+        offset = len(self._sizes)
+        self._sizes.extend(int(x) for x in index.sizes)
+        self._doc_idx.extend(int(x) for x in (offset + index.doc_idx)[1:])
+        with open(data_file_path(another_prefix), "rb") as f:
+            shutil.copyfileobj(f, self._data_file)
+
     def finalize(self, index_file):
         self._data_file.close()
         MMapIndex.write(index_file, self._dtype, self._sizes, self._doc_idx)
+
+
+def split_list(lst, n):
+    """n nearly equal consecutive parts (data_utils.py:258-264)."""
+    k, m = divmod(len(lst), n)
+    return [lst[i * k + min(i, m):(i + 1) * k + min(i + 1, m)] for i in range(n)]
+
+
+def encode_tokenised_line(json_line):
+    """Default `encode`: a line that already holds its token ids."""
+    meta = json.loads(json_line)
+    return {"input_ids": torch.as_tensor(meta["input_ids"], dtype=torch.int64)}
+
+
+def _build_one_cache(encode, vocab_size, json_files, cache_prefix, cache_worker):
+    """data_utils.py:333-385: one document per non-empty encoded line, in file and line order."""
+    if os.path.exists(data_file_path(cache_prefix)) and os.path.exists(index_file_path(cache_prefix)):
+        return 0
+    if os.path.exists(data_file_path(cache_prefix)):
+        raise RuntimeError("%s.bin already exists. Please manually remove it first" % cache_prefix)
+    builder = MMapIndexedDatasetBuilder(data_file_path(cache_prefix), dtype=best_fitting_dtype(vocab_size))
+    items = 0
+    for jsf in json_files:
+        with open(jsf, "r", encoding="utf-8") as fin:
+            if cache_worker and cache_worker > 1:
+                with Pool(cache_worker) as pool:
+                    encoded = list(pool.imap(encode, fin, 25))
+            else:
+                encoded = [encode(line) for line in fin]
+        for meta in encoded:
+            ids = torch.as_tensor(meta["input_ids"]).int().cpu().numpy()
+            if ids.size == 0:
+                continue
+            builder.add_item(ids)
+            builder.end_document()
+            items += 1
+    builder.finalize(index_file_path(cache_prefix))
+    return items
+
+
+def build_data_cache(encode, vocab_size, json_file, cache_prefix, cache_worker=4, cache_splits=1, cache_indices=None):
+    """Token cache `<cache_prefix>.idx/.bin` from line-json files (data_utils.py:268-330).  With cache_splits > 1 the files
+    (or, for a single file, its lines) are cut into that many parts, each built as `<cache_prefix>_<i>` -- only the parts
+    named in cache_indices, when given -- and, when all were built, merged in order into one cache."""
+    assert cache_splits >= 1
+    json_file = list(json_file) if isinstance(json_file, (list, tuple)) else [json_file]
+    if cache_splits == 1:
+        return _build_one_cache(encode, vocab_size, json_file, cache_prefix, cache_worker)
+    temp_files = []
+    if len(json_file) == 1:
+        with open(json_file[0], "r", encoding="utf-8") as f:
+            lines = f.readlines()
+        assert len(lines) >= cache_splits
+        json_file = []
+        for part in split_list(lines, cache_splits):
+            with tempfile.NamedTemporaryFile(mode="w+", delete=False) as tf:
+                tf.writelines(part)
+                json_file.append(tf.name)
+                temp_files.append(tf.name)
+    cache_splits = min(len(json_file), cache_splits)
+    parts = split_list(json_file, cache_splits)
+    items = 0
+    try:
+        for i, part in enumerate(parts):
+            if cache_indices is not None and i not in cache_indices:
+                continue
+            items += _build_one_cache(encode, vocab_size, part, cache_prefix + "_%d" % i, cache_worker)
+    finally:
+        for name in temp_files:
+            os.remove(name)
+    if cache_indices is None:
+        merged = MMapIndexedDatasetBuilder(data_file_path(cache_prefix), dtype=best_fitting_dtype(vocab_size))
+        for i in range(len(parts)):
+            merged.merge_file_(cache_prefix + "_%d" % i)
+        merged.finalize(index_file_path(cache_prefix))
+    return items
 
 
 def num_epochs_for(tokens_per_epoch, seq_length, num_samples):
@@ -227,3 +318,36 @@ class MMapIndexDataset(torch.utils.data.Dataset):
             cu = get_cu_seqlens(input_ids, self.eos_token_id)
             results.update({"cu_seqlens": torch.LongTensor(cu), "position_ids": torch.LongTensor(get_position_ids(cu))})
         return results
+
+
+class MMapIndexJsonDataset(MMapIndexDataset):
+    """The reference's `mmap_index_json` dataset (nlp_dataset.py:322-395): builds the token cache under
+    `<data_root>/<cache_dir>/<cache_prefix>` from `json_file` when it does not exist yet, then serves packed samples from it.
+
+    tokenizer: any object with `vocab_size` and `eos_token_id`.  transformer: a callable `meta -> {'input_ids': ...}` applied
+    to each parsed json line (the reference builds it from its parser registry, which is outside this build); without one
+    the lines must already hold `input_ids`.  Only the native sample-location builder exists, so `cache_location_builder`
+    is accepted and ignored."""
+
+    def __init__(self, data_root, seed, total_samples, max_seq_length, json_file=None, json_type="line", tokenizer=None,
+                 transformer=None, cache_dir="train_data_cache", cache_prefix="mmap_sentebnse", cache_worker=4,
+                 cache_skip_warmup=True, cache_log_freq=100, cache_splits=1, cache_location_builder="py", ignore_index=-100,
+                 cutoff_last_epoch=0.95, with_cu_lens=False):
+        self.tokenizer = tokenizer
+        self.transformer = transformer
+        self.ignore_index = ignore_index
+        prefix = os.path.join(data_root, cache_dir, cache_prefix)
+        if not (os.path.exists(index_file_path(prefix)) and os.path.exists(data_file_path(prefix))):
+            os.makedirs(os.path.join(data_root, cache_dir), exist_ok=True)
+            assert json_file is not None, ("you have not a cache .bin&.idx file of cache_prefix: {}, you must provide as least "
+                                           "one json file to generate them".format(prefix))
+            assert json_type == "line", "Only support line type json to build the cache .bin&.idx file"
+            build_data_cache(self.data_encode, getattr(tokenizer, "vocab_size", None), json_file, prefix, cache_worker,
+                             cache_splits=cache_splits)
+        super().__init__(prefix, seed, total_samples, max_seq_length, eos_token_id=getattr(tokenizer, "eos_token_id", None),
+                         cutoff_last_epoch=cutoff_last_epoch, with_cu_lens=with_cu_lens)
+
+    def data_encode(self, json_line):
+        if self.transformer is None:
+            return encode_tokenised_line(json_line)
+        return self.transformer(json.loads(json_line))

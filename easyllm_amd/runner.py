@@ -3,8 +3,8 @@
 Counterpart of `BaseRunner.forward_step` -> DeepSpeed `train_batch` (llm/runners/base_llm_runner.py:236-245)
 for what lies inside this build: `loss = loss_fn(model(inputs), labels); loss.backward()`, weight
 gradients landing in fp32 `main_grad` buffers (DeepSpeed's bf16 optimizer accumulates in fp32).
-The optimizer step, gradient clipping, loss scaling by accumulation steps and ZeRO are DeepSpeed's
-and are not reproduced.
+The optimizer step with global-norm clipping that follows lives in optimizer.py; loss scaling by the
+number of accumulation steps and ZeRO partitioning are DeepSpeed's and are not reproduced.
 """
 import torch
 
@@ -76,8 +76,16 @@ class GraphedStep:
         self._accumulate = accumulate
         self._pending_flag = None
 
+        grads = [p for p in model.parameters() if getattr(p, "main_grad", None) is not None]
+        # The eager warm-up passes of an accumulating capture add the capture batch's gradients to the buffers; keep what
+        # the buffers (and their "fresh" marks) held and put it back once the graph exists.
+        saved = [(p.main_grad.clone(), getattr(p, "main_grad_fresh", False)) for p in grads] if accumulate else None
+
         def one_step():
-            if not accumulate:
+            if accumulate:
+                for p in grads:  # every captured gradient kernel must add: no buffer may be marked fresh here
+                    p.main_grad_fresh = False
+            else:
                 zero_main_grads(model)
             return forward_step(model, self.inputs, self.labels)
 
@@ -96,6 +104,12 @@ class GraphedStep:
             self.loss = one_step()
         self._flags = list(functional.CAPTURED_ID_FLAGS)
         del functional.CAPTURED_ID_FLAGS[:]
+        if saved is not None:
+            torch.cuda.synchronize()
+            for p, (buf, fresh) in zip(grads, saved):
+                p.main_grad.copy_(buf)
+                p.main_grad_fresh = fresh
+        self._grads = grads
         self._host_flags = [torch.zeros(1, dtype=torch.int32, pin_memory=True) for _ in self._flags]
         self._flag_event = None
 
@@ -113,6 +127,11 @@ class GraphedStep:
             _tree_copy(self.inputs, inputs)
         if labels is not None:
             _tree_copy(self.labels, labels)
+        if self._accumulate:
+            for p in self._grads:  # the graph adds: a buffer marked fresh (zero_main_grads) starts from zero
+                if getattr(p, "main_grad_fresh", False):
+                    p.main_grad.zero_()
+                    p.main_grad_fresh = False
         self.graph.replay()
         for host, (flag, _) in zip(self._host_flags, self._flags):
             host.copy_(flag, non_blocking=True)

@@ -58,11 +58,14 @@ int ezl_rope_apply(const void* x, void* out, const void* cos_table, const void* 
 /* ---- token embedding: base_modules/layers/vocab_parallel_emb.py:106-137 (F.embedding, TP=1) ----
  * gather: out[r] = weight[ids[r]] (bit-exact row copy); an id outside [0, vocab) ORs 1 (id >= vocab)
  * or 2 (id < 0) into *bad_flag (device int32) and yields a zero row.
- * scatter_add: dweight_f32[id] += sum of dy[r] over rows with ids[r] == id, fp32, no atomics, fixed (row) order. */
+ * scatter_add: dweight_f32[id] += sum of dy[r] over rows with ids[r] == id, fp32, added in increasing row order whatever
+ * the launch does (bit-reproducible), in time linear in `rows`; workspace: ezl_embed_scatter_add_workspace_bytes(rows, vocab)
+ * bytes of device memory, 4-byte aligned, contents irrelevant before and after. */
 int ezl_embed_gather(const void* ids, const void* weight, void* out, void* bad_flag, int64_t rows, int64_t h, int64_t vocab,
                      void* stream);
-int ezl_embed_scatter_add(const void* ids, const void* dy, void* dweight_f32, int64_t rows, int64_t h, int64_t vocab,
-                          void* stream);
+int64_t ezl_embed_scatter_add_workspace_bytes(int64_t rows, int64_t vocab);
+int ezl_embed_scatter_add(const void* ids, const void* dy, void* dweight_f32, void* workspace, int64_t workspace_bytes,
+                          int64_t rows, int64_t h, int64_t vocab, void* stream);
 
 /* ---- layout / dtype plumbing of llama/llama.py:145-188 (transpose, undo, float16_to_fp32) ---- */
 int ezl_transpose01(const void* x, void* y, int64_t d0, int64_t d1, int64_t inner, void* stream); /* y[j,i,:] = x[i,j,:] */

@@ -24,6 +24,8 @@ against library routines, closed forms and invariants:
   packed inputs ........ pinned (hand-worked known answers)
   sample locations ..... pinned (the reference's own helpers.cpp compiled into oracle/_ref by oracle/build_ref.py, and
                                 slicing the concatenated token stream by brute force)
+  bf16-storage mode .... pinned (storage off is bit-identical to the fp32 functions; the rounding helper equals
+                                ``x.bfloat16().float()`` in both directions; a linear chain worked by hand)
   optimizer step ....... pinned (``torch.optim.AdamW`` over several steps with and without weight decay,
                                 ``torch.nn.utils.clip_grad_norm_``); apex / DeepSpeed themselves are absent, so
                                 their rounding order inside the update is parity unpinned
@@ -41,6 +43,31 @@ import numpy as np
 import torch
 
 IGNORE_INDEX = -100  # llm/data/nlp_dataset.py:20
+
+
+# --------------------------------------------------------------------------------------------
+# storage rounding of the reference's bf16 path
+# --------------------------------------------------------------------------------------------
+class _RoundTrip(torch.autograd.Function):
+    """Rounds a tensor to `dtype` and back, and does the same to the gradient that flows back through
+    it: a tensor the reference materialises in bf16 has a bf16 gradient as well."""
+
+    @staticmethod
+    def forward(ctx, x, dtype):
+        ctx.dtype = dtype
+        return x.to(dtype).to(x.dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        return g.to(ctx.dtype).to(g.dtype), None
+
+
+def stored(x, storage_dtype=None):
+    """`x` as the reference's 16-bit path holds it in memory: all arithmetic stays in the dtype of `x`
+    (fp32), only the result is rounded to `storage_dtype` (None: no rounding, `x` itself is returned)."""
+    if storage_dtype is None:
+        return x
+    return _RoundTrip.apply(x, storage_dtype)
 
 
 # --------------------------------------------------------------------------------------------
@@ -187,30 +214,43 @@ def swiglu_bwd(gate, up, dout):
 # --------------------------------------------------------------------------------------------
 # J. decoder layer   (llama/transformer.py:410-491,595; :756-802)
 # --------------------------------------------------------------------------------------------
-def decoder_layer(x, W, prefix, cfg, position_ids=None, cu_seqlens=None):
-    """x [s, b, h] -> [s, b, h].  W maps state-dict names (llama/utils.py:158-210) to tensors."""
+def decoder_layer(x, W, prefix, cfg, position_ids=None, cu_seqlens=None, storage_dtype=None):
+    """x [s, b, h] -> [s, b, h].  W maps state-dict names (llama/utils.py:158-210) to tensors.
+
+    storage_dtype=torch.bfloat16 rounds every tensor that the reference's bf16 path writes to memory -- the output of
+    each norm (fused_layer_norm.py:56-57), of each linear (column_parallel_linear.py:42, row_parallel_linear.py:113),
+    of the rotation (positional_embeddings.py:121), of the attention seam (transformer.py:106-115), of silu and of its
+    product with `up` (transformer.py:220-222) and of both residual adds (:786, :797) -- and their gradients, while the
+    arithmetic that produces each of them stays fp32.  The rotary tables stay fp32 (the reference rounds them too,
+    positional_embeddings.py:33-35; the kernels under test do not)."""
+    st = lambda t: stored(t, storage_dtype)  # noqa: E731
     s, b, h = x.shape
     nq, nk, d = cfg["num_attention_heads"], cfg["num_kv_attention_heads"], cfg["head_dim"]
     eps = cfg.get("eps", 1e-6)
-    a = rmsnorm(x, W[prefix + "input_layernorm.weight"], eps)  # :766
+    a = st(rmsnorm(x, W[prefix + "input_layernorm.weight"], eps))  # :766
     if (prefix + "self_attn.wqkv.weight") in W:  # qkv_pack, :426-429 (q | k | v along the output dim)
-        qkv = linear(a, W[prefix + "self_attn.wqkv.weight"], W.get(prefix + "self_attn.wqkv.bias"))
+        qkv = st(linear(a, W[prefix + "self_attn.wqkv.weight"], W.get(prefix + "self_attn.wqkv.bias")))
         q, k, v = qkv[..., : nq * d], qkv[..., nq * d: (nq + nk) * d], qkv[..., (nq + nk) * d:]
     else:
-        q = linear(a, W[prefix + "self_attn.q_proj.weight"], W.get(prefix + "self_attn.q_proj.bias"))  # :422
-        k = linear(a, W[prefix + "self_attn.k_proj.weight"], W.get(prefix + "self_attn.k_proj.bias"))
-        v = linear(a, W[prefix + "self_attn.v_proj.weight"], W.get(prefix + "self_attn.v_proj.bias"))
+        q = st(linear(a, W[prefix + "self_attn.q_proj.weight"], W.get(prefix + "self_attn.q_proj.bias")))  # :422
+        k = st(linear(a, W[prefix + "self_attn.k_proj.weight"], W.get(prefix + "self_attn.k_proj.bias")))
+        v = st(linear(a, W[prefix + "self_attn.v_proj.weight"], W.get(prefix + "self_attn.v_proj.bias")))
     pos = positions_sb(s, b, position_ids)  # [s, b]
     cos, sin = rope_cos_sin(pos, d, cfg.get("rope_base", 10000.0), dtype=x.dtype)  # [s, b, d]
-    q = apply_rope(q.reshape(s, b, nq, d), cos[:, :, None, :], sin[:, :, None, :])  # :437-448
-    k = apply_rope(k.reshape(s, b, nk, d), cos[:, :, None, :], sin[:, :, None, :])
+    q = st(apply_rope(q.reshape(s, b, nq, d), cos[:, :, None, :], sin[:, :, None, :]))  # :437-448
+    k = st(apply_rope(k.reshape(s, b, nk, d), cos[:, :, None, :], sin[:, :, None, :]))
     v = v.reshape(s, b, nk, d)
-    ctx = attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), cu_seqlens)  # :475-490
+    ctx = st(attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), cu_seqlens))  # :475-490
     ctx = ctx.transpose(0, 1).reshape(s, b, nq * d)  # :491
-    x1 = x + linear(ctx, W[prefix + "self_attn.o_proj.weight"])  # :595, :786
-    m = rmsnorm(x1, W[prefix + "post_attention_layernorm.weight"], eps)  # :787
-    act = swiglu(linear(m, W[prefix + "mlp.gate_proj.weight"]), linear(m, W[prefix + "mlp.up_proj.weight"]))
-    return x1 + linear(act, W[prefix + "mlp.down_proj.weight"])  # :789-797
+    x1 = st(x + st(linear(ctx, W[prefix + "self_attn.o_proj.weight"])))  # :595, :786
+    m = st(rmsnorm(x1, W[prefix + "post_attention_layernorm.weight"], eps))  # :787
+    gate = st(linear(m, W[prefix + "mlp.gate_proj.weight"]))
+    up = st(linear(m, W[prefix + "mlp.up_proj.weight"]))
+    if storage_dtype is None:
+        act = swiglu(gate, up)
+    else:
+        act = st(st(torch.nn.functional.silu(gate)) * up)  # glu_activations.py:56-61 then transformer.py:222
+    return st(x1 + st(linear(act, W[prefix + "mlp.down_proj.weight"])))  # :789-797
 
 
 # --------------------------------------------------------------------------------------------
@@ -220,22 +260,24 @@ def layer_prefix(i):
     return "%d." % (i + 3)  # specs 0 cast, 1 embedding, 2 transpose, 3.. layers
 
 
-def model_forward(W, cfg, tokens, position_ids=None, cu_seqlens=None):
+def model_forward(W, cfg, tokens, position_ids=None, cu_seqlens=None, storage_dtype=None):
     """tokens i64 [b, s] -> fp32 logits [b, s, V].
 
     With no cu_seqlens (3-tuple input) the reference drops position_ids and the mask after the
     embedding (word_embedings.py:169-172): positions are arange(s) and attention is purely causal.
+    storage_dtype: see decoder_layer; the logits are rounded as well (lm_head.py:62 produces bf16, llama.py:187-188
+    widens them again for the loss).
     """
     L = cfg["num_layers"]
     if cu_seqlens is None:
         position_ids = None
-    x = embedding(tokens, W["1.word_embeddings.weight"])  # [b, s, h]
+    x = stored(embedding(tokens, W["1.word_embeddings.weight"]), storage_dtype)  # [b, s, h]
     x = x.transpose(0, 1).contiguous()  # llama.py:157-168
     for i in range(L):
-        x = decoder_layer(x, W, layer_prefix(i), cfg, position_ids, cu_seqlens)
+        x = decoder_layer(x, W, layer_prefix(i), cfg, position_ids, cu_seqlens, storage_dtype)
     x = x.transpose(0, 1).contiguous()  # :175-179
-    x = rmsnorm(x, W["%d.weight" % (L + 4)], cfg.get("eps", 1e-6))  # :182
-    return linear(x, W["%d.word_embeddings.weight" % (L + 5)])  # lm_head.py:62, untied
+    x = stored(rmsnorm(x, W["%d.weight" % (L + 4)], cfg.get("eps", 1e-6)), storage_dtype)  # :182
+    return stored(linear(x, W["%d.word_embeddings.weight" % (L + 5)]), storage_dtype)  # lm_head.py:62, untied
 
 
 def init_weights(cfg, seed, sigma=0.02, dtype=torch.float32, round_to_bf16=False):

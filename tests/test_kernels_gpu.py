@@ -151,6 +151,29 @@ def test_embedding_scatter_add(K, gpu_device, V, h, shape):
     assert torch.equal(dW2, dW)
 
 
+def test_embedding_scatter_add_packed_batch_with_frequent_tokens(K, gpu_device):
+    """16384 rows as in the packed workload, ids drawn so that every bucket path runs: most ids once, many a few times
+    (sorted in LDS), one id 700 times and one 3000 times (beyond the LDS sort).  Row-order fp32 sums, bit for bit."""
+    T, V, h = 16384, 32000, 512
+    g = torch.Generator().manual_seed(5)
+    ids = torch.randint(0, V, (T,), generator=g)
+    ids[torch.randperm(T, generator=g)[:3000]] = 17
+    ids[torch.randperm(T, generator=g)[:700]] = 31999
+    ids[torch.randint(0, T, (2000,), generator=g)] = torch.randint(100, 140, (2000,), generator=g)
+    dy = rnd(T, h, seed=11)
+    print("embed scatter, packed batch", flush=True)
+    dW = torch.zeros(V, h, device=gpu_device)
+    K.embed_scatter_add(ids.view(1, T).to(gpu_device), dy.view(1, T, h).to(gpu_device), dW)
+    seq = torch.zeros(V, h)
+    dyf = dy.float()
+    for r, i in enumerate(ids.tolist()):
+        seq[i] += dyf[r]
+    assert torch.equal(dW.cpu(), seq)
+    dW2 = torch.zeros(V, h, device=gpu_device)
+    K.embed_scatter_add(ids.view(1, T).to(gpu_device), dy.view(1, T, h).to(gpu_device), dW2)
+    assert torch.equal(dW2, dW)
+
+
 # ------------------------------------------------------------------------------------- plumbing
 def test_transpose_add_cast_exact(K, gpu_device):
     x = rnd(5, 3, 64, seed=11)
@@ -224,6 +247,72 @@ def test_gemm_linearity_large(K, gpu_device):
     close(y[:64], ref, "gemm big slice")
 
 
+def test_gemm_wrapper_refuses_what_would_read_or_add_out_of_place(K, gpu_device):
+    x, w = rnd(64, 128, seed=1).to(gpu_device), rnd(256, 128, seed=2).to(gpu_device)
+    with pytest.raises(ValueError):
+        K.linear_wgrad(rnd(64, 256, seed=3).to(gpu_device), x, accumulate=True)  # nothing to add to
+    with pytest.raises(ValueError):
+        K.linear_dgrad_multi([rnd(64, 256, seed=3).to(gpu_device)], [w], accumulate=True)
+    with pytest.raises(ValueError):
+        K.gemm(x, w, 128, 256, 128, 128, 128, True, True)  # claims 128 rows of x, there are 64
+    with pytest.raises(ValueError):
+        K.gemm(x, w, 64, 256, 256, 128, 128, True, True)  # reduction longer than the rows
+    with pytest.raises(ValueError):
+        K.gemm(x.float(), w, 64, 256, 128, 128, 128, True, True)
+
+
+def test_gemm_all_forms_at_full_size_reductions(K, gpu_device):
+    """The 7B-shape MLP linears, every form against the fp32 product of the same bf16 operands on the host:
+    forward (K = 4096), input gradient (K = 11008), fp32 weight gradient over K = T = 4096 tokens written and then
+    accumulated, and the input gradient of three linears that share their input as one launch (K = 3 x 4096)."""
+    T, n_in, n_out = 4096, 4096, 11008
+    x, w, dy = rnd(T, n_in, seed=71), rnd(n_out, n_in, seed=72, scale=0.02), rnd(T, n_out, seed=73)
+    xg, wg, dyg = x.to(gpu_device), w.to(gpu_device), dy.to(gpu_device)
+    xf, wf, dyf = x.float(), w.float(), dy.float()
+    print("gemm full size: forward", flush=True)
+    close(K.linear_fwd(xg, wg), xf @ wf.t(), "gemm fwd 4096x11008x4096")
+    print("gemm full size: dgrad", flush=True)
+    close(K.linear_dgrad(dyg, wg), dyf @ wf, "gemm dgrad 4096x4096x11008")
+    print("gemm full size: wgrad fp32", flush=True)
+    rdw = dyf.t() @ xf
+    mg = torch.empty(n_out, n_in, dtype=torch.float32, device=gpu_device)
+    K.linear_wgrad(dyg, xg, out=mg, accumulate=False)
+    close(mg, rdw, "gemm wgrad fp32 11008x4096x4096", rel=2e-3, cos=0.999999)
+    K.linear_wgrad(dyg, xg, out=mg, accumulate=True)
+    close(mg, 2 * rdw, "gemm wgrad fp32 accumulated twice", rel=2e-3, cos=0.999999)
+    close(K.linear_wgrad(dyg, xg), rdw, "gemm wgrad bf16 11008x4096x4096")
+    print("gemm full size: dgrad over q/k/v", flush=True)
+    ws = [rnd(4096, n_in, seed=74 + i, scale=0.02) for i in range(3)]
+    dys = [rnd(T, 4096, seed=77 + i) for i in range(3)]
+    ref = sum(a.float() @ b.float() for a, b in zip(dys, ws))
+    close(K.linear_dgrad_multi([a.to(gpu_device) for a in dys], [b.to(gpu_device) for b in ws]), ref,
+          "gemm dgrad over three linears, K = 12288")
+
+
+def test_gemm_operand_beyond_two_to_the_31_elements(K, gpu_device):
+    """d logits of a packed 16384-token batch over a 152064-entry vocabulary is 2.5e9 elements (5 GB): the input gradient
+    (that matrix as the row operand) and the weight gradient (as the transposed operand) must address all of it.
+    Checked on the first and last rows / columns against fp32 on the host."""
+    T, V, h = 16384, 152064, 256
+    print("gemm, operand of %.2e elements" % (T * V), flush=True)
+    torch.manual_seed(91)
+    dy = torch.empty(T, V, dtype=torch.bfloat16, device=gpu_device)
+    for r0 in range(0, T, 2048):  # filled in pieces: the generator's fp32 temporaries stay small
+        dy[r0:r0 + 2048] = torch.randn(2048, V, device=gpu_device).bfloat16()
+    w = (torch.randn(V, h, device=gpu_device) * 0.02).bfloat16()
+    x = torch.randn(T, h, device=gpu_device).bfloat16()
+    dx = K.linear_dgrad(dy, w)
+    rows = torch.cat([torch.arange(0, 8), torch.arange(T // 2 - 4, T // 2 + 4), torch.arange(T - 8, T)])
+    close(dx[rows.to(gpu_device)], dy[rows.to(gpu_device)].float().cpu() @ w.float().cpu(), "dgrad rows of a 5 GB operand")
+    dw = torch.empty(V, h, dtype=torch.float32, device=gpu_device)
+    K.linear_wgrad(dy, x, out=dw)
+    cols = torch.cat([torch.arange(0, 8), torch.arange(V // 2 - 4, V // 2 + 4), torch.arange(V - 8, V)])
+    ref = dy[:, cols.to(gpu_device)].float().cpu().t() @ x.float().cpu()
+    close(dw[cols.to(gpu_device)], ref, "wgrad rows from a 5 GB operand", rel=2e-3)
+    del dy, dw
+    torch.cuda.empty_cache()
+
+
 # ------------------------------------------------------------------------------------- attention
 def _attn_case(K, dev, s, b, nq, nk, d, cu, seed):
     q, k, v, do = rnd(s, b, nq, d, seed=seed), rnd(s, b, nk, d, seed=seed + 1), rnd(s, b, nk, d, seed=seed + 2), rnd(s, b, nq, d, seed=seed + 3)
@@ -259,6 +348,34 @@ def test_attention_varlen_across_batch_rows(K, gpu_device):
     _attn_case(K, gpu_device, 256, 2, 4, 4, 128, cu, 40)
 
 
+@pytest.mark.parametrize("s,nq,nk", [(4096, 2, 2), (4096, 8, 1)])
+def test_attention_at_full_sequence_length(K, gpu_device, s, nq, nk):
+    """seq 4096, d 128: 64 key tiles of online softmax per query block, MHA and a GQA group of 8 (the 70B shape's group),
+    forward and backward against the fp32 oracle."""
+    print("attention full length", s, nq, nk, flush=True)
+    _attn_case(K, gpu_device, s, 1, nq, nk, 128, None, 50)
+
+
+def test_attention_64_query_heads_on_8_kv_heads(K, gpu_device):
+    """The 70B head layout (64 q / 8 kv): with a multiple of 8 kv heads the workgroup renumbering deals whole kv heads to
+    the 8 L2 domains; short sequence so that the host finishes quickly."""
+    print("attention 64q/8kv", flush=True)
+    _attn_case(K, gpu_device, 320, 1, 64, 8, 128, None, 60)
+    _attn_case(K, gpu_device, 200, 2, 64, 8, 128, None, 61)
+
+
+def test_attention_packed_16k_tokens(K, gpu_device):
+    """The packed workload's token count and document recipe (16384 tokens, lengths log-uniform in [64, 4096]) on 2 heads:
+    block-diagonal causal attention over ~17 documents, forward and backward against the oracle."""
+    lens = O.packed_doc_lengths(16384, 64, 4096, 1005)
+    cu = [0]
+    for l in lens:
+        cu.append(cu[-1] + l)
+    print("attention packed 16k,", len(lens), "documents", flush=True)
+    _attn_case(K, gpu_device, 16384, 1, 2, 2, 128, cu, 70)
+    _attn_case(K, gpu_device, 16384, 1, 4, 1, 128, cu, 71)
+
+
 def test_attention_forward_with_drifting_and_jumping_maxima(K, gpu_device):
     """The forward kernel moves the reference point of its exponentials only when a row's maximum has outgrown it by a
     factor 2^8.  Scores here grow along the keys: slowly for most rows (many tiles pass between two moves, probabilities
@@ -287,7 +404,14 @@ def test_attention_forward_with_drifting_and_jumping_maxima(K, gpu_device):
 # ------------------------------------------------------------------------------------- cross entropy
 @pytest.mark.parametrize("rows,V,dtype,cut", [(33, 32000, torch.bfloat16, 0), (5, 152064, torch.bfloat16, 0),
                                               (17, 4096, torch.float32, 0), (9, 32000, torch.float32, 0),
-                                              (12, 1024, torch.bfloat16, 24)])
+                                              (12, 1024, torch.bfloat16, 24),
+                                              # rows kept on chip in LDS + registers (one read of the logits): more rows than
+                                              # blocks, so every block walks several rows and refills its slots; a row length
+                                              # whose last register vector is mostly past the end; cut columns; and the lengths
+                                              # either side of that kernel's range
+                                              (300, 152064, torch.bfloat16, 0), (270, 73736, torch.bfloat16, 0),
+                                              (40, 152064, torch.bfloat16, 64), (6, 180224, torch.bfloat16, 0),
+                                              (6, 73720, torch.bfloat16, 0), (6, 180232, torch.bfloat16, 0)])
 def test_cross_entropy_all_paths(K, gpu_device, rows, V, dtype, cut):
     print("ce", rows, V, dtype, cut, flush=True)
     g = torch.Generator().manual_seed(50)

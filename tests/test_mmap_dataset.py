@@ -118,3 +118,80 @@ def test_dataset_samples_are_windows_of_the_document_stream(tmp_path):
     assert M.num_epochs_for(100, 10, 9) == 1 and M.num_epochs_for(100, 10, 10) == 2  # (100 - 1) // 10 = 9 samples per epoch
     with pytest.raises(FileNotFoundError):
         M.MMapIndexDataset(str(tmp_path / "missing"), 1, 1, 8)
+
+
+class _Tok:
+    vocab_size, eos_token_id = 1000, 2
+
+    def __len__(self):
+        return 1001  # the collator pads with len(tokenizer) - 1
+
+
+def _write_json(path, docs):
+    import json
+    with open(path, "w") as f:
+        for d in docs:
+            f.write(json.dumps({"input_ids": d}) + "\n")
+
+
+def test_cache_built_from_json_lines_equals_the_cache_built_from_token_arrays(tmp_path):
+    rng = np.random.RandomState(7)
+    docs = [rng.randint(3, 1000, size=int(rng.randint(1, 50))).tolist() + [2] for _ in range(23)]
+    docs.insert(5, [])  # an empty document is skipped (data_utils.py:372-373)
+    _write_json(tmp_path / "a.jsonl", docs[:10])
+    _write_json(tmp_path / "b.jsonl", docs[10:])
+    direct = _write_cache(tmp_path, [d for d in docs if d])
+    for workers, splits, name in ((1, 1, "one"), (2, 1, "pool"), (1, 2, "split_files")):
+        prefix = str(tmp_path / name)
+        n = M.build_data_cache(M.encode_tokenised_line, 1000, [str(tmp_path / "a.jsonl"), str(tmp_path / "b.jsonl")], prefix,
+                               cache_worker=workers, cache_splits=splits)
+        assert n == 23
+        for ext in (".idx", ".bin"):
+            assert open(prefix + ext, "rb").read() == open(direct + ext, "rb").read(), (name, ext)
+    # a single file split by lines into three parts, built part by part, merged
+    _write_json(tmp_path / "all.jsonl", docs)
+    prefix = str(tmp_path / "split_lines")
+    M.build_data_cache(M.encode_tokenised_line, 1000, str(tmp_path / "all.jsonl"), prefix, cache_worker=1, cache_splits=3)
+    for ext in (".idx", ".bin"):
+        assert open(prefix + ext, "rb").read() == open(direct + ext, "rb").read()
+    assert M.split_list(list(range(7)), 3) == [[0, 1, 2], [3, 4], [5, 6]]
+    with pytest.raises(RuntimeError):  # a stray .bin without its .idx is never overwritten
+        open(str(tmp_path / "stray.bin"), "wb").close()
+        M.build_data_cache(M.encode_tokenised_line, 1000, str(tmp_path / "a.jsonl"), str(tmp_path / "stray"), cache_worker=1)
+
+
+def test_json_dataset_builds_its_cache_once_and_feeds_the_collator(tmp_path):
+    from easyllm_amd import data as D
+    rng = np.random.RandomState(11)
+    docs = [rng.randint(3, 1000, size=int(rng.randint(2, 40))).tolist() + [2] for _ in range(60)]
+    _write_json(tmp_path / "train.jsonl", docs)
+    seq = 64
+    kw = dict(data_root=str(tmp_path), seed=5, total_samples=8, max_seq_length=seq, tokenizer=_Tok(), cache_worker=1,
+              with_cu_lens=True)
+    ds = M.MMapIndexJsonDataset(json_file=str(tmp_path / "train.jsonl"), **kw)
+    assert os.path.exists(str(tmp_path / "train_data_cache" / "mmap_sentebnse.idx"))
+    again = M.MMapIndexJsonDataset(**kw)  # the cache exists: no json needed
+    assert torch.equal(ds[3]["input_ids"], again[3]["input_ids"])
+    with pytest.raises(AssertionError):
+        M.MMapIndexJsonDataset(str(tmp_path / "elsewhere"), 5, 8, seq, tokenizer=_Tok())
+    # a transformer that maps parsed json to tokens is applied per line
+    doubled = M.MMapIndexJsonDataset(json_file=str(tmp_path / "train.jsonl"), cache_prefix="doubled",
+                                     transformer=lambda meta: {"input_ids": torch.tensor(meta["input_ids"] * 2)}, **kw)
+    assert doubled._index.sizes.tolist() == [2 * len(d) for d in docs]
+    # collator: next-token shift, boundaries clamped to the sequence length and flattened over the batch
+    items = [ds[0], ds[1]]
+    batch = D.batch_align_collate(items, pad_token_id=1000, max_seq_length=seq, pretrain=True)
+    for b, it in enumerate(items):
+        assert batch["input_ids"][b].tolist() == it["input_ids"][:-1].tolist()
+        assert batch["labels"][b].tolist() == it["input_ids"][1:].tolist()
+        assert batch["position_ids"][b].tolist() == it["position_ids"][:-1].tolist()
+    want = O.flatten_cu_seqlens([it["cu_seqlens"].tolist() for it in items], seq)
+    assert batch["cu_seqlens"].tolist() == want.tolist() and batch["cu_seqlens"][-1].item() == 2 * seq
+    (tokens, pos, mask, cu), (labels, loss_mask) = D.flash_batch_from(batch, pad_token_id=1000, pretrain=True)
+    assert mask.all() and loss_mask.dtype == torch.bool and torch.equal(cu, batch["cu_seqlens"])
+    # ragged items without the packed fields: padded with the pad token / ignore index to the longest, shifted
+    short = {"input_ids": torch.tensor([5, 6, 7]), "labels": torch.tensor([5, 6, 7])}
+    long_ = {"input_ids": torch.tensor([8, 9, 10, 11, 12]), "labels": torch.tensor([8, 9, 10, 11, 12])}
+    b2 = D.batch_align_collate([short, long_], pad_token_id=1000, max_seq_length=seq, alignment=4)
+    assert b2["input_ids"].tolist() == [[5, 6, 1000, 1000, 1000, 1000, 1000, 1000], [8, 9, 10, 11, 1000, 1000, 1000, 1000]]
+    assert b2["labels"].tolist() == [[6, 7, -100, -100, -100, -100, -100, -100], [9, 10, 11, 12, -100, -100, -100, -100]]

@@ -133,6 +133,38 @@ def test_batched_mha_with_bool_loss_mask_and_accumulation(gpu_device):
         close(p.main_grad, 2 * one[n], "accumulated " + n, rel=1e-3)
 
 
+def test_packed_samples_from_the_token_cache_through_the_step(gpu_device, tmp_path):
+    """The data path of the packed workload end to end: a token cache on disk built from tokenised json lines ->
+    `MMapIndexJsonDataset(with_cu_lens=True)` samples (llm/data/nlp_dataset.py:596-646) -> `BatchAlignCollector`'s shift
+    and boundary flattening (nlp_dataloader.py:131-187) -> `flash_batch_pipe`'s tuple (nlp_batch_fn.py:181-205) -> the HIP
+    step; loss, logits and every gradient against the oracle fed the same batch."""
+    import json
+    import numpy as np
+    from easyllm_amd import data as D, mmap_dataset as M
+    V, pad, eos, seq, b = 1008, 1007, 2, 256, 2
+
+    class Tok:
+        vocab_size, eos_token_id = V, eos
+
+    rng = np.random.RandomState(21)
+    with open(tmp_path / "train.jsonl", "w") as f:
+        for _ in range(80):
+            f.write(json.dumps({"input_ids": rng.randint(3, 1000, size=int(rng.randint(5, 120))).tolist() + [eos]}) + "\n")
+    ds = M.MMapIndexJsonDataset(str(tmp_path), seed=9, total_samples=6, max_seq_length=seq, json_file=str(tmp_path / "train.jsonl"),
+                                tokenizer=Tok(), cache_worker=1, with_cu_lens=True)
+    items = [ds[1], ds[4]]
+    batch = D.batch_align_collate(items, pad_token_id=pad, max_seq_length=seq, pretrain=True)
+    inputs, (labels, loss_mask) = D.flash_batch_from(batch, pad_token_id=pad, pretrain=True)
+    tokens, position_ids, attention_mask, cu_seqlens = inputs
+    assert tuple(tokens.shape) == (b, seq) and cu_seqlens[-1].item() == b * seq and len(cu_seqlens) > 4
+    assert position_ids[0, :5].tolist() == [0, 1, 2, 3, 4] and (position_ids == 0).sum().item() == len(cu_seqlens) - 1
+    w = dict(num_layers=2, hidden_size=512, num_attention_heads=8, num_kv_attention_heads=2, intermediate_size=1024,
+             vocab_size=V, seq=seq, batch=b, seed=31)
+    model, Wt = build_pair(w, gpu_device)
+    print("step on packed samples of a token cache:", len(cu_seqlens) - 1, "documents", flush=True)
+    check_step(model, Wt, w, inputs, labels, loss_mask, gpu_device)
+
+
 def test_loss_paths_agree_and_reference_api(gpu_device):
     from easyllm_amd.losses import CrossEntropy, vocab_parallel_cross_entropy
     g = torch.Generator().manual_seed(9)

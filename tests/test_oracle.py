@@ -245,6 +245,131 @@ def test_model_packed_documents_are_independent():
     assert torch.allclose(packed, torch.cat([a, c], 1), atol=1e-5)
 
 
+# ---------------------------------------------------------------- bf16-storage mode
+def _bf(t):
+    return t.bfloat16().float()
+
+
+def test_storage_rounding_helper_rounds_values_and_gradients():
+    x = torch.tensor([1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, -3.3333, 1e-3], requires_grad=True)
+    y = O.stored(x, torch.bfloat16)
+    assert torch.equal(y, _bf(x.detach()))
+    assert y[0].item() == 1.0 and y[1].item() == 1.0 + 2.0 ** -6  # ties go to the even mantissa
+    g = torch.tensor([0.1, 1.0 + 2.0 ** -8, 7.77, -2.0 ** -20])
+    y.backward(g)
+    assert torch.equal(x.grad, _bf(g))
+    assert O.stored(x, None) is x
+
+
+def test_storage_chain_worked_by_hand():
+    """y = st(st(x * a) * b), loss = sum(y * c): every rounding point of values and gradients written out."""
+    torch.manual_seed(5)
+    x, a, b, c = (torch.randn(64) for _ in range(4))
+    xg = x.clone().requires_grad_(True)
+    y = O.stored(O.stored(xg * a, torch.bfloat16) * b, torch.bfloat16)
+    (y * c).sum().backward()
+    t1 = _bf(x * a)
+    assert torch.equal(y.detach(), _bf(t1 * b))
+    g_outer = _bf(c)                 # gradient of the outer stored tensor
+    g_inner = _bf(g_outer * b)       # gradient of the inner stored tensor
+    assert torch.equal(xg.grad, g_inner * a)
+    assert not torch.equal(xg.grad, c * b * a)
+
+
+def _small_model(seed=9):
+    cfg = dict(num_layers=2, hidden_size=64, num_attention_heads=4, num_kv_attention_heads=2, head_dim=16,
+               intermediate_size=96, vocab_size=128)
+    W = O.init_weights(cfg, seed=seed, sigma=0.1, round_to_bf16=True)
+    g = torch.Generator().manual_seed(seed)
+    tokens = torch.randint(0, 128, (2, 24), generator=g)
+    labels = torch.randint(0, 128, (2, 24), generator=g)
+    return cfg, W, tokens, labels
+
+
+def _loss_and_grads(cfg, W, tokens, labels, storage, **kw):
+    Wg = {k_: v.clone().requires_grad_(True) for k_, v in W.items()}
+    logits = O.model_forward(Wg, cfg, tokens, storage_dtype=storage, **kw)
+    loss = O.cross_entropy_loss(logits, labels, torch.ones(labels.shape))
+    loss.backward()
+    return logits.detach(), loss.item(), {k_: v.grad for k_, v in Wg.items()}
+
+
+def test_storage_off_is_the_fp32_oracle_bit_for_bit():
+    """A round trip through fp32 changes nothing, so the storage-mode code path (every `stored` call, the two-step
+    silu * up) must reproduce the plain fp32 functions exactly, gradients included; so must a packed batch."""
+    cfg, W, tokens, labels = _small_model()
+    for kw in ({}, dict(position_ids=torch.tensor([O.get_position_ids([0, 10, 24])] * 2),
+                        cu_seqlens=torch.tensor([0, 10, 24, 34, 48]))):
+        l0, loss0, g0 = _loss_and_grads(cfg, W, tokens, labels, None, **kw)
+        l1, loss1, g1 = _loss_and_grads(cfg, W, tokens, labels, torch.float32, **kw)
+        assert torch.equal(l0, l1) and loss0 == loss1
+        for k_ in g0:
+            assert torch.equal(g0[k_], g1[k_]), k_
+
+
+def test_storage_bf16_stays_near_fp32_and_near_transformers_bf16():
+    """The bf16-storage result is a perturbation of the fp32 one of the size of bf16 rounding (not zero, not large), its
+    logits are bf16 numbers, and it sits as close to transformers' LlamaForCausalLM run in bf16 -- library code that
+    stores the same tensors in bf16 -- as that model sits to its own fp32 run."""
+    from transformers import LlamaConfig, LlamaForCausalLM
+    cfg, W, tokens, labels = _small_model()
+    l0, loss0, g0 = _loss_and_grads(cfg, W, tokens, labels, None)
+    l1, loss1, g1 = _loss_and_grads(cfg, W, tokens, labels, torch.bfloat16)
+    assert torch.equal(l1, _bf(l1)) and not torch.equal(l0, l1)
+    rel = ((l1 - l0).norm() / l0.norm()).item()
+    assert 1e-4 < rel < 2e-2, rel
+    assert abs(loss1 - loss0) < 1e-2 * loss0
+    for k_ in g0:
+        r = ((g1[k_] - g0[k_]).norm() / g0[k_].norm()).item()
+        assert r < 5e-2, (k_, r)
+    hf_cfg = LlamaConfig(vocab_size=128, hidden_size=64, intermediate_size=96, num_hidden_layers=2,
+                         num_attention_heads=4, num_key_value_heads=2, rms_norm_eps=1e-6, rope_theta=10000.0,
+                         max_position_embeddings=64, tie_word_embeddings=False, attention_bias=False,
+                         hidden_act="silu", attn_implementation="eager")
+    hf = LlamaForCausalLM(hf_cfg).float().eval()
+    sd = {"model.embed_tokens.weight": W["1.word_embeddings.weight"], "model.norm.weight": W["6.weight"],
+          "lm_head.weight": W["7.word_embeddings.weight"]}
+    for i in range(2):
+        for n in ("input_layernorm.weight", "self_attn.q_proj.weight", "self_attn.k_proj.weight", "self_attn.v_proj.weight",
+                  "self_attn.o_proj.weight", "post_attention_layernorm.weight", "mlp.gate_proj.weight",
+                  "mlp.up_proj.weight", "mlp.down_proj.weight"):
+            sd["model.layers.%d.%s" % (i, n)] = W["%d.%s" % (i + 3, n)]
+    hf.load_state_dict(sd, strict=False)
+    with torch.no_grad():
+        hf32 = hf(input_ids=tokens).logits
+        hf16 = hf.bfloat16()(input_ids=tokens).logits.float()
+    gap_lib = ((hf16 - hf32).norm() / hf32.norm()).item()
+    gap_ours = ((l1 - hf16).norm() / hf32.norm()).item()
+    assert gap_ours < 2.0 * gap_lib, (gap_ours, gap_lib)
+
+
+def test_storage_rounding_decorrelates_evaluations_that_differ_only_in_summation_precision():
+    """Why a bf16-storage evaluation is a noise floor and not a trajectory: the same stack, the same rounding points, once
+    with fp32 and once with fp64 arithmetic between them.  Without storage rounding the two agree to 1e-6; with it, a
+    difference of 1e-7 before a rounding flips the rounded value with probability ~ difference / ulp, each flip is a whole
+    ulp, and a handful of ops later the two evaluations are almost as far from each other as each is from the unrounded
+    result.  (So a correct bf16 implementation can be required to stay within the floor's distance of fp32, not to land
+    on any particular bf16-storage result.)"""
+    cfg = dict(num_layers=4, hidden_size=512, num_attention_heads=8, num_kv_attention_heads=8, head_dim=64,
+               intermediate_size=1376, vocab_size=2000)
+    W = O.init_weights(cfg, seed=1, round_to_bf16=True)
+    W64 = {k_: v.double() for k_, v in W.items()}
+    tokens = torch.randint(0, 2000, (1, 256), generator=torch.Generator().manual_seed(2))
+
+    def dist(a, b):
+        return ((a.double() - b.double()).norm() / b.double().norm()).item()
+
+    with torch.no_grad():
+        f32 = O.model_forward(W, cfg, tokens)
+        f64 = O.model_forward(W64, cfg, tokens)
+        s32 = O.model_forward(W, cfg, tokens, storage_dtype=torch.bfloat16)
+        s64 = O.model_forward(W64, cfg, tokens, storage_dtype=torch.bfloat16)
+    assert dist(f32, f64) < 1e-5
+    floor = dist(s32, f64)
+    assert 2e-3 < floor < 2e-2 and abs(dist(s64, f64) - floor) < 0.1 * floor
+    assert dist(s32, s64) > 0.7 * floor
+
+
 # ---------------------------------------------------------------- cross entropy
 def test_cross_entropy_matches_library():
     logits = torch.randn(2, 9, 40) * 3

@@ -1,23 +1,27 @@
-"""Full-size runs of the benchmark workloads (C2..C5) checked through size-independent properties:
+"""Full-size runs of the benchmark workloads (C2..C5) checked through size-independent properties (the whole-step
+comparison of C2..C4 with the oracle is in test_full_size_parity_gpu.py):
 
-* causality: the logits of the first 64 positions (of the first document) depend only on those 64 tokens, so
-  the CPU oracle evaluated on that prefix with the same weights must reproduce them;
 * the fused loss equals the reference-composed loss path on the same logits and sits in [ln V, ln V + 3]
   for random N(0, 0.02) weights;
-* activation recompute changes nothing: loss and gradients are bit-identical for any number of
-  checkpointed layers (C5, dynamic checkpoint rule);
-* gradient accumulation over two identical micro-batches doubles the fp32 main gradients.
+* gradient accumulation over two identical micro-batches doubles the fp32 main gradients;
+* C5 exactly as specified (8 layers, 16384 packed tokens, its own size_map => the first 4 layers recomputed):
+  activation recompute changes nothing -- loss and gradients are bit-identical for 4, 0 and 8 recomputed layers;
+* causality and document independence (C5): the logits of the first positions of a document depend only on those
+  tokens, so the oracle evaluated on that prefix alone must reproduce them (rule of tests/_parity.py: the stated bar
+  against the fp32 oracle, or -- eight bf16-stored layers deep -- no farther from it than the oracle's own
+  bf16-storage evaluation is).
 """
 import math
 
 import pytest
 import torch
 
+import _parity as P
 from oracle import llama_oracle as O
 
 pytestmark = pytest.mark.gpu
 
-PREFIX = 64
+PREFIX = 256
 
 
 def _oracle_cfg(w):
@@ -38,16 +42,6 @@ def _close(a, ref, name, rel=2e-2, cos=0.9999, l2=None):
         assert r <= l2, "%s: relative L2 error %.3e" % (name, r)
 
 
-def _close_logits(a, ref, name):
-    """Logits of a full-size stack: every intermediate is stored in bf16 (as in the reference's bf16 path), and the
-    rounding accumulates with depth -- measured against the fp32 oracle at the 7B shape the relative L2 error
-    is 0.17 % after the first RMSNorm, 0.55 % after the first attention block, 0.95 / 1.3 / 1.6 / 1.8 % after
-    layers 1..4, i.e. cosine 0.9998 on the logits, with no single kernel off (each one meets 2e-2 / 0.9999 on its
-    own in test_kernels_gpu.py, and so does the 2-layer C1 model).  Bounds here: cosine >= 0.9995, relative L2
-    <= 2.5e-2, max error <= 5e-2 of max |ref| (a 5-sigma event over millions of elements)."""
-    _close(a, ref, name, rel=5e-2, cos=0.9995, l2=2.5e-2)
-
-
 def _run(name, dev, layers=None):
     from easyllm_amd import runner, workloads as W
     w = dict(W.WORKLOADS[name])
@@ -60,11 +54,16 @@ def _run(name, dev, layers=None):
     return w, model, inputs, labels, doc_lens
 
 
-def _prefix_check(w, model, inputs, logits, doc_lens):
-    n = PREFIX if doc_lens is None else min(PREFIX, doc_lens[0])
+def _prefix_check(w, model, tokens, logits, start, length, name):
+    n = min(PREFIX, length)
     Wt = {k: v.detach().float().cpu() for k, v in model.state_dict().items() if "inv_freq" not in k}
-    ref = O.model_forward(Wt, _oracle_cfg(w), inputs[0][:1, :n].cpu())
-    _close_logits(logits[0, :n], ref[0], "prefix logits")
+    ids = tokens[:1, start:start + n].cpu()
+    ref = O.model_forward(Wt, _oracle_cfg(w), ids)
+    rep = P.Report("C5")
+    rep.check(name, logits[0, start:start + n], ref[0],
+              lambda: O.model_forward(Wt, _oracle_cfg(w), ids, storage_dtype=torch.bfloat16)[0])
+    print("\n".join(rep.lines), flush=True)
+    assert not rep.failures, "\n".join(rep.failures)
 
 
 @pytest.mark.parametrize("name,layers", [("C2", None), ("C3", None), ("C4", None)])
@@ -75,7 +74,6 @@ def test_full_size_step_properties(gpu_device, name, layers):
     w, model, inputs, labels, doc_lens = _run(name, gpu_device, layers)
     logits = model(inputs)
     assert logits.dtype == torch.bfloat16 and tuple(logits.shape) == (w["batch"], w["seq"], w["vocab_size"])
-    _prefix_check(w, model, inputs, logits.detach(), doc_lens)
     plain = CrossEntropy(is_prefix=False, fused=False)(logits.detach(), labels).item()
     loss = model.loss_fn(logits, labels)
     lnv = math.log(w["vocab_size"])
@@ -94,28 +92,34 @@ def test_full_size_step_properties(gpu_device, name, layers):
 
 
 def test_packed_dynamic_checkpoint_full_size(gpu_device):
-    """C5 at full token count (16384 packed tokens, 7B shape) with 4 instead of 8 layers to keep the test short:
-    recompute-forward must not change a single bit, and documents must be independent of each other."""
+    """C5 as specified: 8 layers, 16384 packed tokens, size_map {4096: 0, 8192: 2, 16384: 4, 32768: 8} => the rule picks
+    k = 4 by itself.  Recompute-forward must not change a single bit (k = 4, 0, 8), and documents must be independent
+    of each other."""
     from easyllm_amd import runner
     print("workload C5", flush=True)
-    w, model, inputs, labels, doc_lens = _run("C5", gpu_device, layers=4)
-    assert sum(doc_lens) == 16384
+    w, model, inputs, labels, doc_lens = _run("C5", gpu_device)
+    assert sum(doc_lens) == 16384 and w["num_layers"] == 8
+    assert model.size_map == {4096: 0, 8192: 2, 16384: 4, 32768: 8}
+    names = ("4.self_attn.q_proj.weight", "6.mlp.gate_proj.weight", "10.mlp.down_proj.weight", "1.word_embeddings.weight")
+    params = dict(model.named_parameters())
     results = []
-    for k in (2, 0, 4):
-        model.size_map = {16384: k}
+    for k in (4, 0, 8):
+        if k != 4:
+            model.size_map = {16384: k}
         runner.zero_main_grads(model)
         loss = runner.forward_step(model, inputs, labels)
         assert model.recompute_count == k
-        results.append((loss.item(), dict(model.named_parameters())["4.self_attn.q_proj.weight"].main_grad.clone(),
-                        dict(model.named_parameters())["6.mlp.gate_proj.weight"].main_grad.clone()))
+        results.append((loss.item(), [params[n].main_grad.clone() for n in names]))
+        print("C5 k=%d loss %.6f" % (k, loss.item()), flush=True)
     for other in results[1:]:
         assert other[0] == results[0][0]
-        assert torch.equal(other[1], results[0][1]) and torch.equal(other[2], results[0][2])
+        for a, b in zip(other[1], results[0][1]):
+            assert torch.equal(a, b)
+    lnv = math.log(w["vocab_size"])
+    assert lnv <= results[0][0] <= lnv + 3.0
     with torch.no_grad():
         logits = model(inputs)
-    _prefix_check(w, model, inputs, logits, doc_lens)
-    # second document: same logits as running that document alone from position 0
-    a, e = doc_lens[0], doc_lens[0] + min(PREFIX, doc_lens[1])
-    Wt = {k: v.detach().float().cpu() for k, v in model.state_dict().items() if "inv_freq" not in k}
-    ref = O.model_forward(Wt, _oracle_cfg(w), inputs[0][:1, a:e].cpu())
-    _close_logits(logits[0, a:e], ref[0], "second document logits")
+    _prefix_check(w, model, inputs[0], logits, 0, doc_lens[0], "first document logits")
+    # a later document: same logits as running that document alone from position 0
+    i = max(range(1, len(doc_lens)), key=lambda j: min(doc_lens[j], PREFIX) * 100000 - j)
+    _prefix_check(w, model, inputs[0], logits, sum(doc_lens[:i]), doc_lens[i], "document %d logits" % i)
