@@ -33,6 +33,8 @@ SIGNATURES = {
     "ezl_attn_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64p, _vp],
     "ezl_attn_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32,
                      _i64p, _vp],
+    "ezl_mask_compact": [_vp, _i64, _i64, _vp, _vp, _vp, _vp],
+    "ezl_rows_gather": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     "ezl_ce_prepare": [_vp, _vp, _i32, _i64, _vp, _vp, _i64, _vp],
     "ezl_ce_fwd": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],
     "ezl_ce_bwd": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _vp],

@@ -278,6 +278,70 @@ __global__ __launch_bounds__(kBlock) void embed_scatter_bucket_kernel(const int6
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Unpadding by a key-padding mask (FlashAttention.forward, llama/transformer.py:117-141: unpad_input / pad_input)
+// ---------------------------------------------------------------------------------------------
+// mask [rows, s_len] (non-zero = keep), flattened to n = rows * s_len tokens.  One block walks the tokens 1024 at a time
+// with a running count:  idx[p] = flat index of the p-th kept token (entries past the last kept token: -1),
+// inv[i] = position of token i among the kept ones, or -1;  cu[r + 1] = kept tokens in rows 0..r (cu[0] = 0).
+__global__ __launch_bounds__(1024) void mask_compact_kernel(const unsigned char* __restrict__ mask, int64_t n, int s_len,
+                                                            int* __restrict__ idx, int* __restrict__ inv, int* __restrict__ cu) {
+    __shared__ int wsum[16];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    int base = 0;
+    if (tid == 0) cu[0] = 0;
+    for (int64_t i0 = 0; i0 < n; i0 += 1024) {
+        const int64_t i = i0 + tid;
+        const int m = (i < n && mask[i]) ? 1 : 0;
+        int incl = m;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += v;
+        }
+        __syncthreads();  // wsum of the previous round has been read
+        if (lane == 63) wsum[wv] = incl;
+        __syncthreads();
+        int before = 0, total = 0;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            before += k < wv ? wsum[k] : 0;
+            total += wsum[k];
+        }
+        const int upto = base + before + incl;  // kept tokens among 0..i
+        if (i < n) {
+            inv[i] = m ? upto - 1 : -1;
+            if (m) idx[upto - 1] = (int)i;
+            if ((i + 1) % s_len == 0) cu[(i + 1) / s_len] = upto;
+        }
+        base += total;
+    }
+    for (int64_t i = base + tid; i < n; i += 1024) idx[i] = -1;
+}
+
+// out row r = src row idx[r] (zeros where idx[r] is negative or past the source); a row number maps to memory as
+// (r / s_len) * batch_stride + (r % s_len) * seq_stride on either side, so [s, b, ...] activations are read and
+// written where they lie.
+__global__ __launch_bounds__(kBlock) void rows_gather_kernel(const bf16_t* __restrict__ src, const int* __restrict__ idx,
+                                                             bf16_t* __restrict__ out, int64_t n_out, int width, int64_t n_src,
+                                                             int src_s_len, int64_t src_ss, int64_t src_sb, int out_s_len,
+                                                             int64_t out_ss, int64_t out_sb) {
+    const int w8 = width >> 3;
+    for (int64_t r = blockIdx.x; r < n_out; r += gridDim.x) {
+        const int64_t j = idx[r];
+        const bool ok = j >= 0 && j < n_src;
+        const bf16_t* s = src + (ok ? (j / src_s_len) * src_sb + (j % src_s_len) * src_ss : 0);
+        bf16_t* o = out + (r / out_s_len) * out_sb + (r % out_s_len) * out_ss;
+        for (int c = threadIdx.x; c < w8; c += kBlock) {
+            bf16x8 v;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[k] = (bf16_t)0.0f;
+            if (ok) v = ld_bf16x8(s + c * 8);
+            st_bf16x8(o + c * 8, v);
+        }
+    }
+}
+
 // y[j, i, :] = x[i, j, :]  for x [d0, d1, inner]   (llama/llama.py:157-168,175-179)
 __global__ __launch_bounds__(kBlock) void transpose01_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ y, int64_t d0,
                                                              int64_t d1, int inner) {
@@ -541,5 +605,32 @@ extern "C" int ezl_bias_grad(const void* dy, void* db_bf16, void* db_f32, int ac
     hipLaunchKernelGGL(ezl_colsum_kernel<0>, dim3((unsigned)((n + 63) / 64)), dim3(kColsumThreads), 0, (hipStream_t)stream,
                        (const float*)workspace, 64, (int)n, (bf16_t*)db_bf16, (float*)db_f32, accumulate);
     EZL_LAUNCH_CHECK("ezl_bias_grad(colsum)");
+    return EZL_OK;
+}
+
+extern "C" int ezl_mask_compact(const void* mask_u8, int64_t rows, int64_t s_len, void* idx, void* inv, void* cu_seqlens, void* stream) {
+    EZL_REQUIRE(rows >= 0 && s_len > 0 && rows * s_len < (1LL << 31), EZL_EINVAL, "ezl_mask_compact: bad shape");
+    EZL_REQUIRE(cu_seqlens && (rows == 0 || (mask_u8 && idx && inv)), EZL_EINVAL, "ezl_mask_compact: null pointer");
+    hipLaunchKernelGGL(mask_compact_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const unsigned char*)mask_u8, rows * s_len,
+                       (int)s_len, (int*)idx, (int*)inv, (int*)cu_seqlens);
+    EZL_LAUNCH_CHECK("ezl_mask_compact");
+    return EZL_OK;
+}
+
+extern "C" int ezl_rows_gather(const void* src, const void* idx, void* out, int64_t n_out, int64_t width, int64_t n_src,
+                               int64_t src_s_len, int64_t src_seq_stride, int64_t src_batch_stride, int64_t out_s_len,
+                               int64_t out_seq_stride, int64_t out_batch_stride, void* stream) {
+    EZL_REQUIRE(n_out >= 0 && n_src >= 0 && width > 0 && width % 8 == 0 && width < (1LL << 31), EZL_EUNSUPPORTED,
+                "ezl_rows_gather: width must be a multiple of 8");
+    EZL_REQUIRE(src_s_len > 0 && out_s_len > 0 && src_s_len < (1LL << 31) && out_s_len < (1LL << 31) && src_seq_stride % 8 == 0 &&
+                    src_batch_stride % 8 == 0 && out_seq_stride % 8 == 0 && out_batch_stride % 8 == 0,
+                EZL_EINVAL, "ezl_rows_gather: strides must be multiples of 8 elements");
+    EZL_REQUIRE((n_out == 0 || (idx && out && (src || n_src == 0))) && ezl_aligned16(src) && ezl_aligned16(out), EZL_EINVAL,
+                "ezl_rows_gather: null or misaligned pointer");
+    if (n_out == 0) return EZL_OK;
+    hipLaunchKernelGGL(rows_gather_kernel, dim3(grid_for(n_out, 1)), dim3(kBlock), 0, (hipStream_t)stream, (const bf16_t*)src,
+                       (const int*)idx, (bf16_t*)out, n_out, (int)width, n_src, (int)src_s_len, src_seq_stride, src_batch_stride,
+                       (int)out_s_len, out_seq_stride, out_batch_stride);
+    EZL_LAUNCH_CHECK("ezl_rows_gather");
     return EZL_OK;
 }

@@ -236,21 +236,23 @@ extern "C" int64_t ezl_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t h) {
     return (int64_t)256 * h * (int64_t)sizeof(float);
 }
 
-extern "C" int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const void* rstd,
-                               const void* dresidual, void* dx, void* dw_bf16, void* dw_f32, int accumulate,
-                               void* workspace, int64_t workspace_bytes, int64_t rows, int64_t h, void* stream) {
-    EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h <= 8192, EZL_EUNSUPPORTED,
-                "ezl_rmsnorm_bwd: need h %% 8 == 0 and h <= 8192 (got h=%lld)", (long long)h);
-    EZL_REQUIRE(weight && workspace && (rows == 0 || (dy && x && rstd && dx)), EZL_EINVAL, "ezl_rmsnorm_bwd: null pointer");
-    EZL_REQUIRE((dw_bf16 != nullptr) != (dw_f32 != nullptr), EZL_EINVAL,
-                "ezl_rmsnorm_bwd: exactly one of dw_bf16 / dw_f32");
-    EZL_REQUIRE(workspace_bytes >= ezl_rmsnorm_bwd_workspace_bytes(rows, h), EZL_EINVAL,
-                "ezl_rmsnorm_bwd: workspace too small");
-    EZL_REQUIRE(ezl_aligned16(dy) && ezl_aligned16(x) && ezl_aligned16(weight) && ezl_aligned16(dx) &&
-                    ezl_aligned16(dresidual),
-                EZL_EINVAL, "ezl_rmsnorm_bwd: pointers must be 16-byte aligned");
-    EZL_REQUIRE(rows < (1LL << 31), EZL_EUNSUPPORTED, "ezl_rmsnorm_bwd: too many rows");
-    hipStream_t st = (hipStream_t)stream;
+namespace {
+
+int rmsnorm_bwd_check(const char* name, const void* dy, const void* x, const void* weight, const void* rstd, const void* dresidual,
+                      const void* dx, const void* dw_bf16, const void* dw_f32, int64_t rows, int64_t h) {
+    EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h <= 8192, EZL_EUNSUPPORTED, "%s: need h %% 8 == 0 and h <= 8192 (got h=%lld)",
+                name, (long long)h);
+    EZL_REQUIRE(weight && (rows == 0 || (dy && x && rstd && dx)), EZL_EINVAL, "%s: null pointer", name);
+    EZL_REQUIRE((dw_bf16 != nullptr) != (dw_f32 != nullptr), EZL_EINVAL, "%s: exactly one of dw_bf16 / dw_f32", name);
+    EZL_REQUIRE(ezl_aligned16(dy) && ezl_aligned16(x) && ezl_aligned16(weight) && ezl_aligned16(dx) && ezl_aligned16(dresidual),
+                EZL_EINVAL, "%s: pointers must be 16-byte aligned", name);
+    EZL_REQUIRE(rows < (1LL << 31), EZL_EUNSUPPORTED, "%s: too many rows", name);
+    return EZL_OK;
+}
+
+// both entry points: `partials` holds one fp32 row of h per block (at most 256 blocks), every used row fully written
+int rmsnorm_bwd_launch(const void* dy, const void* x, const void* weight, const void* rstd, const void* dresidual, void* dx,
+                       void* dw_bf16, void* dw_f32, int accumulate, float* partials, int64_t rows, int64_t h, hipStream_t st) {
     const int tpr = tpr_for((int)h);
     const int nchunk = ((int)h + tpr * 8 - 1) / (tpr * 8);
     const int rpb = 1024 / tpr;
@@ -261,7 +263,7 @@ extern "C" int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight
 #define LAUNCH(NC, DR)                                                                                            \
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<NC, DR>), dim3((unsigned)grid), dim3(1024), smem, st, (const bf16_t*)dy, \
                        (const bf16_t*)x, (const bf16_t*)weight, (const float*)rstd, (const bf16_t*)dresidual,     \
-                       (bf16_t*)dx, (float*)workspace, (int)rows, (int)h, tpr)
+                       (bf16_t*)dx, partials, (int)rows, (int)h, tpr)
     if (dresidual) {
         if (nchunk == 1) LAUNCH(1, true); else if (nchunk == 2) LAUNCH(2, true); else LAUNCH(4, true);
     } else {
@@ -269,8 +271,20 @@ extern "C" int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight
     }
 #undef LAUNCH
     EZL_LAUNCH_CHECK("ezl_rmsnorm_bwd");
-    hipLaunchKernelGGL(ezl_colsum_kernel<0>, dim3((unsigned)((h + 63) / 64)), dim3(kColsumThreads), 0, st, (const float*)workspace,
+    hipLaunchKernelGGL(ezl_colsum_kernel<0>, dim3((unsigned)((h + 63) / 64)), dim3(kColsumThreads), 0, st, (const float*)partials,
                        (int)grid, (int)h, (bf16_t*)dw_bf16, (float*)dw_f32, accumulate);
     EZL_LAUNCH_CHECK("ezl_rmsnorm_bwd(colsum)");
     return EZL_OK;
+}
+
+}  // namespace
+
+extern "C" int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const void* rstd,
+                               const void* dresidual, void* dx, void* dw_bf16, void* dw_f32, int accumulate,
+                               void* workspace, int64_t workspace_bytes, int64_t rows, int64_t h, void* stream) {
+    if (const int rc = rmsnorm_bwd_check("ezl_rmsnorm_bwd", dy, x, weight, rstd, dresidual, dx, dw_bf16, dw_f32, rows, h)) return rc;
+    EZL_REQUIRE(workspace && workspace_bytes >= ezl_rmsnorm_bwd_workspace_bytes(rows, h), EZL_EINVAL,
+                "ezl_rmsnorm_bwd: workspace missing or too small");
+    return rmsnorm_bwd_launch(dy, x, weight, rstd, dresidual, dx, dw_bf16, dw_f32, accumulate, (float*)workspace, rows, h,
+                              (hipStream_t)stream);
 }

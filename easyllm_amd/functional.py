@@ -260,6 +260,38 @@ def flash_attention(q, k, v, cu_seqlens=None, scale=None):
     return FlashAttnFunction.apply(q, k, v, cu_seqlens, scale)
 
 
+class RowsGatherFunction(torch.autograd.Function):
+    """x [s, b, heads, d] -> [s', b', heads, d] whose rows (in (b s) order) are x's rows picked by `idx` (zeros where idx
+    is negative).  `idx_back` is the inverse selection: the gradient is the same gather the other way round.  With the
+    indices of `kernels.mask_compact` this is unpad_input / pad_input of llama/transformer.py:121-141."""
+
+    @staticmethod
+    def forward(ctx, x, idx, idx_back, out_sb):
+        ctx.save_for_backward(idx_back)
+        ctx.in_sb = (x.shape[0], x.shape[1])
+        return K.rows_gather(x, idx, out_sb)
+
+    @staticmethod
+    def backward(ctx, dy):
+        (idx_back,) = ctx.saved_tensors
+        if dy.stride(3) != 1 or dy.stride(2) != dy.shape[3]:
+            dy = dy.contiguous()
+        return K.rows_gather(dy, idx_back, ctx.in_sb), None, None, None
+
+
+def flash_attention_unpadded(q, k, v, key_padding_mask, scale=None):
+    """Attention over the tokens a [b, s] key-padding mask keeps (llama/transformer.py:117-141): every batch row is
+    compressed to its kept tokens, which attend causally among themselves; dropped positions come back as zero rows."""
+    s, b = q.shape[0], q.shape[1]
+    idx, inv, cu = K.mask_compact(key_padding_mask.contiguous())
+    n = s * b
+    qc = RowsGatherFunction.apply(q, idx, inv, (n, 1))
+    kc = RowsGatherFunction.apply(k, idx, inv, (n, 1))
+    vc = RowsGatherFunction.apply(v, idx, inv, (n, 1))
+    oc = FlashAttnFunction.apply(qc, kc, vc, cu, scale)
+    return RowsGatherFunction.apply(oc, inv, idx, (s, b))
+
+
 # --------------------------------------------------------------------------------------------
 # embedding: base_modules/layers/vocab_parallel_emb.py:106-137
 # --------------------------------------------------------------------------------------------

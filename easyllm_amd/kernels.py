@@ -354,6 +354,33 @@ def attn_bwd(q, k, v, out, dout, lse, cu_seqlens=None, scale=None):
     return dq, dk, dv
 
 
+# ------------------------------------------------------------------------------------- unpadding
+def mask_compact(mask):
+    """mask [b, s] (bool / uint8, non-zero = keep) -> (idx int32 [b*s], inv int32 [b*s], cu_seqlens int32 [b+1])."""
+    _need(mask.is_cuda and mask.dim() == 2 and mask.dtype in (torch.bool, torch.uint8) and mask.is_contiguous(),
+          "key padding mask must be a contiguous bool / uint8 [b, s] GPU tensor")
+    b, s = mask.shape
+    idx = torch.empty(b * s, dtype=torch.int32, device=mask.device)
+    inv = torch.empty(b * s, dtype=torch.int32, device=mask.device)
+    cu = torch.empty(b + 1, dtype=torch.int32, device=mask.device)
+    _lib.call("ezl_mask_compact", _p(mask), b, s, _p(idx), _p(inv), _p(cu), _stream())
+    return idx, inv, cu
+
+
+def rows_gather(src, idx, out_shape_sb):
+    """src [s, b, heads, d] (token strides arbitrary) read as rows in (b s) order; out [s', b', heads, d] contiguous whose
+    row r (in (b' s') order) is src row idx[r], or zeros where idx[r] < 0."""
+    _need(idx.is_cuda and idx.dtype == torch.int32 and idx.is_contiguous(), "idx must be a contiguous int32 GPU vector")
+    s, b, nh, d = src.shape
+    so, bo = out_shape_sb
+    _need(idx.numel() == so * bo, "one index per output row")
+    ss, sb = _tok_strides(src, b)
+    out = torch.empty((so, bo, nh, d), dtype=BF16, device=src.device)
+    os_, ob = _tok_strides(out, bo)
+    _lib.call("ezl_rows_gather", _p(src), _p(idx), _p(out), so * bo, nh * d, s * b, s, ss, sb, so, os_, ob, _stream())
+    return out
+
+
 # ------------------------------------------------------------------------------------- cross entropy
 _MASK_DTYPES = {torch.float32: 1, torch.bool: 2, torch.uint8: 2, torch.int64: 3, BF16: 4}
 

@@ -44,15 +44,16 @@ class FlashAttention(torch.nn.Module):
 
     def forward_sb(self, q, k, v, key_padding_mask=None, cu_seqlens=None):
         """Same on [s, b, heads, d] tensors; returns contiguous [s, b, nq, d]."""
-        if key_padding_mask is not None:
-            raise NotImplementedError("unpadding by key_padding_mask is not part of the llama step "
-                                      "(the reference passes cu_seqlens or no mask, transformer.py:480-490)")
         if not self.causal:
             raise NotImplementedError("only causal attention is built")
         if self.training and self.dropout_p != 0.0:
             raise NotImplementedError("attention dropout is 0 in every llama config")
         if q.dtype != torch.bfloat16:
             raise TypeError("the HIP attention computes in bf16")
+        if key_padding_mask is not None:  # :117-141: unpad, attend among the kept tokens of each row, pad back with zeros
+            if tuple(key_padding_mask.shape) != (q.shape[1], q.shape[0]):
+                raise ValueError("key_padding_mask must be [b, s]")
+            return F_.flash_attention_unpadded(q, k, v, key_padding_mask.bool(), self.softmax_scale)
         if cu_seqlens is not None:
             cu_seqlens = cu_seqlens.view(-1).int()  # :103
         return F_.flash_attention(q, k, v, cu_seqlens, self.softmax_scale)
@@ -177,10 +178,14 @@ class ParallelAttention(torch.nn.Module):
         v = value_layer.view(sq, bs, nk, d) if not self.qkv_pack else value_layer.unflatten(-1, (nk, d))
         cos, sin = self.rotary_emb.tables(sq, q.device)
         q, k = apply_rotary_pos_emb(q, k, cos, sin, position_ids)
-        if attention_mask is not None and cu_seqlens is None and attention_mask.dim() == 2:
-            raise NotImplementedError("a 2-D key padding mask without cu_seqlens is not part of the llama step")
+        if attention_mask is None or cu_seqlens is not None:  # :480-488: document boundaries replace the padding mask
+            qk_mask = None
+        elif attention_mask.dim() == 2:
+            qk_mask = attention_mask
+        else:
+            qk_mask = ~attention_mask[:, 0, :, 0]
         with dist_env.get_cuda_rng_tracker().fork():
-            context_layer = self.core_attention_flash.forward_sb(q, k, v, None, cu_seqlens)
+            context_layer = self.core_attention_flash.forward_sb(q, k, v, qk_mask, cu_seqlens)
         context_layer = context_layer.view(sq, bs, nq * d)  # 's b (h d)', already contiguous
         return self.o_proj(context_layer)
 

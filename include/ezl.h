@@ -108,6 +108,18 @@ int ezl_attn_bwd(const void* q, const void* k, const void* v, const void* out, c
                  void* dq, void* dk, void* dv, const void* cu_seqlens, int64_t ndocs, int64_t total_tokens, int64_t s_len,
                  int64_t nq, int64_t nk, int64_t d, float scale, const int64_t* strides, void* stream);
 
+/* ---- unpadding by a key-padding mask: FlashAttention.forward, llama/transformer.py:117-141 (unpad_input / pad_input) ----
+ * mask_compact: mask uint8 / bool [rows, s_len], non-zero = keep.  idx int32 [rows * s_len]: flat index of the p-th kept
+ *   token (-1 past the last one); inv int32 [rows * s_len]: position of each token among the kept ones or -1;
+ *   cu_seqlens int32 [rows + 1]: kept tokens before each row's end (the documents of the unpadded batch).
+ * rows_gather: out row r = src row idx[r], zeros where idx[r] < 0 or >= n_src; rows of `width` bf16; row number n lives at
+ *   (n / s_len) * batch_stride + (n % s_len) * seq_stride elements on either side.  With idx it unpads, with inv it pads
+ *   back (masked positions become zero rows); each is the other's backward. */
+int ezl_mask_compact(const void* mask_u8, int64_t rows, int64_t s_len, void* idx, void* inv, void* cu_seqlens, void* stream);
+int ezl_rows_gather(const void* src, const void* idx, void* out, int64_t n_out, int64_t width, int64_t n_src, int64_t src_s_len,
+                    int64_t src_seq_stride, int64_t src_batch_stride, int64_t out_s_len, int64_t out_seq_stride,
+                    int64_t out_batch_stride, void* stream);
+
 /* ---- loss: base_modules/functions/cross_entropy.py:24-112 and llama/losses.py:20-56 ----
  * logits [rows, vocab] bf16 (dtype 0) or fp32 (dtype 1); labels int64 [rows]; a label outside
  * [0, vocab - cut_size) is masked exactly as the reference does (pred = 0, no one-hot).

@@ -15,7 +15,8 @@ against library routines, closed forms and invariants:
   rope ................. pinned (complex-rotation closed form, relative-position property,
                                 transformers' ``apply_rotary_pos_emb``)
   attention ............ pinned (``F.scaled_dot_product_attention`` causal + GQA, per-document split,
-                                brute-force python loops on tiny inputs)
+                                brute-force python loops on tiny inputs; the key-padding-mask form against a
+                                brute-force loop over kept tokens and, for right-padded rows, the truncated rows)
   swiglu ............... pinned (``F.silu``, closed-form derivative vs autograd)
   layer / model wiring . pinned (``transformers.LlamaForCausalLM`` built from a local config, live and through the
                                 committed fixture tests/golden/hf_llama_tiny.npz: loss, logits, every gradient)
@@ -162,6 +163,20 @@ def positions_sb(s, b, position_ids=None):
 # H / H'. attention   (llama/transformer.py:83-143 semantics, :492-592 definition;
 #                      fused_softmax.py:211-233; base_modules/utils.py:123-125)
 # --------------------------------------------------------------------------------------------
+def attention_unpadded(q, k, v, key_padding_mask, scale=None):
+    """The key_padding_mask branch of FlashAttention.forward (llama/transformer.py:117-141): each batch row is compressed
+    to the tokens its mask keeps (unpad_input), those attend causally among themselves in their compressed order, and the
+    result is scattered back with zero rows at the dropped positions (pad_input).  key_padding_mask: bool [b, s]."""
+    b, s, nq, d = q.shape
+    out = torch.zeros_like(q)
+    for i in range(b):
+        keep = torch.nonzero(key_padding_mask[i]).reshape(-1)
+        if keep.numel() == 0:
+            continue
+        out[i, keep] = attention(q[i:i + 1, keep], k[i:i + 1, keep], v[i:i + 1, keep], None, scale)[0]
+    return out
+
+
 def attention(q, k, v, cu_seqlens=None, scale=None):
     """Causal softmax(q k^T * scale) v.
 

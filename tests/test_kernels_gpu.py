@@ -401,6 +401,50 @@ def test_attention_forward_with_drifting_and_jumping_maxima(K, gpu_device):
     assert torch.allclose(lse.cpu().view(nq, s), ref_lse, rtol=1e-4, atol=2e-3)
 
 
+def test_mask_compaction_is_exact(K, gpu_device):
+    for b, s, seed in ((3, 700, 1), (1, 64, 2), (5, 1500, 3), (2, 8, 4)):
+        mask = torch.rand(b, s, generator=torch.Generator().manual_seed(seed)) < 0.6
+        if b > 2:
+            mask[1] = False  # a row with nothing kept
+            mask[2] = True
+        idx, inv, cu = K.mask_compact(mask.to(gpu_device))
+        flat = mask.reshape(-1)
+        kept = torch.nonzero(flat).reshape(-1)
+        want_idx = torch.full((b * s,), -1, dtype=torch.int32)
+        want_idx[:kept.numel()] = kept.int()
+        want_inv = torch.where(flat, torch.cumsum(flat.int(), 0) - 1, torch.full((b * s,), -1)).int()
+        want_cu = torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(mask.sum(1), 0)]).int()
+        assert torch.equal(idx.cpu(), want_idx) and torch.equal(inv.cpu(), want_inv) and torch.equal(cu.cpu(), want_cu)
+
+
+@pytest.mark.parametrize("s,b,nq,nk,d", [(200, 3, 4, 2, 128), (333, 2, 2, 2, 64)])
+def test_attention_unpadded_by_key_padding_mask(K, gpu_device, s, b, nq, nk, d):
+    """The key_padding_mask branch: gather the kept tokens of every row, attend causally among them, scatter back with zero
+    rows; forward and backward (through the autograd wrappers) against the oracle."""
+    from easyllm_amd.transformer import FlashAttention
+    print("attention unpadded", s, b, nq, nk, d, flush=True)
+    mask = torch.rand(b, s, generator=torch.Generator().manual_seed(7)) < 0.7
+    mask[0, s // 2:] = False  # right padding
+    if b > 2:
+        mask[2] = False       # nothing kept
+    q, k, v, do = rnd(s, b, nq, d, seed=80), rnd(s, b, nk, d, seed=81), rnd(s, b, nk, d, seed=82), rnd(s, b, nq, d, seed=83)
+    qf, kf, vf = [t.float().requires_grad_(True) for t in (q, k, v)]
+    ref = O.attention_unpadded(qf.transpose(0, 1), kf.transpose(0, 1), vf.transpose(0, 1), mask).transpose(0, 1)
+    ref.backward(do.float())
+    qg, kg, vg = [t.to(gpu_device).requires_grad_(True) for t in (q, k, v)]
+    attn = FlashAttention(causal=True)
+    out = attn(qg.transpose(0, 1), kg.transpose(0, 1), vg.transpose(0, 1), key_padding_mask=mask.to(gpu_device)).transpose(0, 1)
+    close(out, ref, "unpadded attn out")
+    dropped = ~mask.t()  # [s, b]
+    assert torch.count_nonzero(out.detach().cpu()[dropped]) == 0
+    out.backward(do.to(gpu_device))
+    close(qg.grad, qf.grad, "unpadded attn dq")
+    close(kg.grad, kf.grad, "unpadded attn dk")
+    close(vg.grad, vf.grad, "unpadded attn dv")
+    for gr in (qg.grad, kg.grad, vg.grad):
+        assert torch.count_nonzero(gr.cpu()[dropped]) == 0
+
+
 # ------------------------------------------------------------------------------------- cross entropy
 @pytest.mark.parametrize("rows,V,dtype,cut", [(33, 32000, torch.bfloat16, 0), (5, 152064, torch.bfloat16, 0),
                                               (17, 4096, torch.float32, 0), (9, 32000, torch.float32, 0),

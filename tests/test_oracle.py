@@ -180,6 +180,40 @@ def test_attention_varlen_equals_independent_documents():
     assert torch.allclose(out, torch.cat([a, c], 1), atol=1e-6)
 
 
+def test_attention_unpadded_by_key_padding_mask():
+    """Kept tokens attend causally among the kept tokens of their own row; dropped positions give zero rows and get no
+    gradient.  Brute force over (row, query, key) on a tiny case; right-padded rows equal the truncated rows."""
+    b, s, nq, nk, d = 3, 9, 4, 2, 8
+    g = torch.Generator().manual_seed(12)
+    q, k, v = torch.randn(b, s, nq, d, generator=g), torch.randn(b, s, nk, d, generator=g), torch.randn(b, s, nk, d, generator=g)
+    mask = torch.tensor([[1, 1, 0, 1, 0, 0, 1, 1, 1], [1] * 9, [0] * 9], dtype=torch.bool)
+    out = O.attention_unpadded(q, k, v, mask)
+    ref = torch.zeros_like(q)
+    for i in range(b):
+        for h in range(nq):
+            hk = h // (nq // nk)
+            for t in range(s):
+                if not mask[i, t]:
+                    continue
+                keys = [u for u in range(t + 1) if mask[i, u]]
+                sc = torch.stack([(q[i, t, h] * k[i, u, hk]).sum() / math.sqrt(d) for u in keys])
+                p = torch.softmax(sc, 0)
+                ref[i, t, h] = sum(p[j] * v[i, u, hk] for j, u in enumerate(keys))
+    assert torch.allclose(out, ref, atol=1e-5)
+    assert torch.count_nonzero(out[2]) == 0 and torch.count_nonzero(out[0, 2]) == 0
+    assert torch.allclose(out[1], O.attention(q[1:2], k[1:2], v[1:2])[0], atol=1e-6)
+    right = torch.zeros(b, s, dtype=torch.bool)
+    right[0, :4] = right[1, :9] = right[2, :1] = True
+    outr = O.attention_unpadded(q, k, v, right)
+    assert torch.allclose(outr[0, :4], O.attention(q[:1, :4], k[:1, :4], v[:1, :4])[0], atol=1e-6)
+    assert torch.allclose(outr[2, 0], v[2, 0].repeat_interleave(nq // nk, 0), atol=1e-6)  # a lone token returns its value
+    qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+    O.attention_unpadded(qg, kg, vg, mask).sum().backward()
+    dropped = ~mask
+    assert torch.count_nonzero(qg.grad[dropped]) == 0 and torch.count_nonzero(kg.grad[dropped]) == 0
+    assert torch.count_nonzero(vg.grad[dropped]) == 0 and torch.count_nonzero(vg.grad[mask]) > 0
+
+
 # ---------------------------------------------------------------- swiglu
 def test_swiglu_and_derivative():
     g = torch.randn(5, 7, dtype=torch.float64, requires_grad=True)
