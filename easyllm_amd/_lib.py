@@ -16,6 +16,7 @@ _vpp = ctypes.POINTER(ctypes.c_void_p)
 SIGNATURES = {
     "ezl_rmsnorm_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp],
     "ezl_rmsnorm_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _i64, _i64, _i64, _vp],
+    "ezl_rmsnorm_bwd_noalloc": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp],
     "ezl_swiglu_fwd": [_vp, _vp, _vp, _i64, _vp],
     "ezl_swiglu_bwd": [_vp, _vp, _vp, _vp, _vp, _i64, _vp],
     "ezl_rope_table": [_vp, _vp, _vp, _i64, _i64, _f32, _vp],
@@ -50,6 +51,7 @@ _SPECIAL = {
     "ezl_version": ([], ctypes.c_int),
     "ezl_last_error": ([], ctypes.c_char_p),
     "ezl_rmsnorm_bwd_workspace_bytes": ([_i64, _i64], _i64),
+    "ezl_rmsnorm_bwd_noalloc_max_h": ([], _i64),
     "ezl_bias_grad_workspace_bytes": ([_i64, _i64], _i64),
     "ezl_embed_scatter_add_workspace_bytes": ([_i64, _i64], _i64),
     "ezl_sumsq_partials": ([], _i64),

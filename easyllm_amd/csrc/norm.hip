@@ -11,6 +11,8 @@
 // row slot through a double-buffered LDS cell (one barrier per row).
 #include "common.h"
 
+#include <mutex>
+
 namespace {
 
 template <int NCHUNK, bool HAS_RES>
@@ -287,4 +289,54 @@ extern "C" int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight
                 "ezl_rmsnorm_bwd: workspace missing or too small");
     return rmsnorm_bwd_launch(dy, x, weight, rstd, dresidual, dx, dw_bf16, dw_f32, accumulate, (float*)workspace, rows, h,
                               (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// ezl_rmsnorm_bwd without a workspace argument, for callers that cannot obtain device memory (code under HIP graph
+// capture, serving loops, harnesses that forbid allocation): the per-block dw partials live in a file-scope device array
+// of the largest size the kernels can need (256 blocks x h <= 8192 floats = 8 MiB), held by every GPU the library runs on
+// until the process ends.  All calls on one GPU share that array: calls that overlap on one GPU (different streams or
+// host threads) race on it.  Nothing in it needs clearing: every row of partials that is read has been written by the
+// same call.
+namespace {
+
+constexpr int kScratchBlocks = 256, kScratchMaxH = 8192;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) float scratch[kScratchBlocks * kScratchMaxH];
+
+// The array's name is only a host-side handle; its device address differs per GPU and is looked up once per device,
+// with that device current.
+float* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+int scratch_for_current_device(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    EZL_REQUIRE(e == hipSuccess && dev >= 0 && dev < kMaxDevices, EZL_EHIP, "ezl_rmsnorm_bwd_noalloc: cannot identify the current device (%s)",
+                hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        EZL_REQUIRE(e == hipSuccess && p, EZL_EHIP, "ezl_rmsnorm_bwd_noalloc: hipGetSymbolAddress failed (%s)", hipGetErrorString(e));
+        g_scratch_ptr[dev] = static_cast<float*>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return EZL_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t ezl_rmsnorm_bwd_noalloc_max_h(void) { return kScratchMaxH; }
+
+extern "C" int ezl_rmsnorm_bwd_noalloc(const void* dy, const void* x, const void* weight, const void* rstd, const void* dresidual,
+                                       void* dx, void* dw_bf16, void* dw_f32, int accumulate, int64_t rows, int64_t h, void* stream) {
+    EZL_REQUIRE(h <= kScratchMaxH, EZL_EUNSUPPORTED, "ezl_rmsnorm_bwd_noalloc: h = %lld exceeds the built-in scratch (h <= %d)",
+                (long long)h, kScratchMaxH);
+    if (const int rc = rmsnorm_bwd_check("ezl_rmsnorm_bwd_noalloc", dy, x, weight, rstd, dresidual, dx, dw_bf16, dw_f32, rows, h)) return rc;
+    EZL_REQUIRE(ezl_rmsnorm_bwd_workspace_bytes(rows, h) <= (int64_t)sizeof(float) * kScratchBlocks * kScratchMaxH, EZL_EUNSUPPORTED,
+                "ezl_rmsnorm_bwd_noalloc: problem exceeds the built-in scratch");
+    float* partials = nullptr;
+    if (const int rc = scratch_for_current_device(&partials)) return rc;
+    return rmsnorm_bwd_launch(dy, x, weight, rstd, dresidual, dx, dw_bf16, dw_f32, accumulate, partials, rows, h, (hipStream_t)stream);
 }

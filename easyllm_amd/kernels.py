@@ -47,8 +47,10 @@ def rmsnorm_fwd(x, weight, eps, residual=None):
     return y, rstd, s
 
 
-def rmsnorm_bwd(dy, x, weight, rstd, dresidual=None, main_grad=None, accumulate=False):
-    """Returns (dx, dw): dw is a bf16 [h] tensor, or None when it was written into main_grad (fp32)."""
+def rmsnorm_bwd(dy, x, weight, rstd, dresidual=None, main_grad=None, accumulate=False, dx=None, dw=None, builtin_scratch=False):
+    """Returns (dx, dw): dw is a bf16 [h] tensor, or None when it was written into main_grad (fp32).
+    builtin_scratch: go through the entry point that keeps its partial sums in the library's own device array; with `dx`
+    (and `dw` when there is no main_grad) passed in, the call then allocates nothing."""
     _bf16c(dy, "dy"); _bf16c(x, "x"); _bf16c(weight, "weight")
     h = x.shape[-1]
     rows = x.numel() // h
@@ -56,14 +58,25 @@ def rmsnorm_bwd(dy, x, weight, rstd, dresidual=None, main_grad=None, accumulate=
     if dresidual is not None:
         _bf16c(dresidual, "dresidual")
         _need(dresidual.shape == x.shape, "dresidual shape mismatch")
-    dx = torch.empty_like(x)
+    if dx is None:
+        dx = torch.empty_like(x)
+    else:
+        _bf16c(dx, "dx")
+        _need(dx.shape == x.shape, "dx shape mismatch")
+    if main_grad is None:
+        if dw is None:
+            dw = torch.empty(h, dtype=BF16, device=x.device)
+        _bf16c(dw, "dw")
+        _need(dw.numel() == h, "dw size mismatch")
+    else:
+        dw = None
+        _need(main_grad.dtype == torch.float32 and main_grad.is_contiguous() and main_grad.numel() == h, "bad main_grad")
+    if builtin_scratch:
+        _lib.call("ezl_rmsnorm_bwd_noalloc", _p(dy), _p(x), _p(weight), _p(rstd), _p(dresidual), _p(dx), _p(dw), _p(main_grad),
+                  1 if accumulate else 0, rows, h, _stream())
+        return dx, dw
     ws_bytes = _lib.rmsnorm_bwd_workspace_bytes(rows, h)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
-    dw = None
-    if main_grad is None:
-        dw = torch.empty(h, dtype=BF16, device=x.device)
-    else:
-        _need(main_grad.dtype == torch.float32 and main_grad.is_contiguous() and main_grad.numel() == h, "bad main_grad")
     _lib.call("ezl_rmsnorm_bwd", _p(dy), _p(x), _p(weight), _p(rstd), _p(dresidual), _p(dx), _p(dw), _p(main_grad),
               1 if accumulate else 0, _p(ws), ws_bytes, rows, h, _stream())
     return dx, dw

@@ -41,6 +41,17 @@ int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const voi
                     void* dw_bf16, void* dw_f32, int accumulate, void* workspace, int64_t workspace_bytes, int64_t rows,
                     int64_t h, void* stream);
 
+/* ezl_rmsnorm_bwd without the workspace argument.  No counterpart in the reference: it exists for callers that cannot
+ * obtain device memory at the call site (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation).  The per-block dw partials go to a device array built into the library (8 MiB per GPU, held until the
+ * process ends), which covers every shape ezl_rmsnorm_bwd accepts (h <= ezl_rmsnorm_bwd_noalloc_max_h() = 8192); a larger
+ * h is refused with EZL_EUNSUPPORTED.  Same kernels and bit-identical results as ezl_rmsnorm_bwd.  All calls on one GPU
+ * share the array: calls that overlap on one GPU (other streams or host threads) race.  The first call on a device looks
+ * the array's address up (hipGetSymbolAddress) and should therefore happen outside a graph capture. */
+int64_t ezl_rmsnorm_bwd_noalloc_max_h(void);
+int ezl_rmsnorm_bwd_noalloc(const void* dy, const void* x, const void* weight, const void* rstd, const void* dresidual, void* dx,
+                            void* dw_bf16, void* dw_f32, int accumulate, int64_t rows, int64_t h, void* stream);
+
 /* ---- SwiGLU: llama/transformer.py:220-222 + base_modules/layers/glu_activations.py:56-61 ---- */
 int ezl_swiglu_fwd(const void* gate, const void* up, void* out, int64_t n, void* stream);
 int ezl_swiglu_bwd(const void* dout, const void* gate, const void* up, void* dgate, void* dup, int64_t n, void* stream);
