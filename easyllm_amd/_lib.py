@@ -21,6 +21,8 @@ SIGNATURES = {
     "ezl_swiglu_bwd": [_vp, _vp, _vp, _vp, _vp, _i64, _vp],
     "ezl_rope_table": [_vp, _vp, _vp, _i64, _i64, _f32, _vp],
     "ezl_rope_apply": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _vp],
+    "ezl_rope_apply_pair": [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp],
+    "ezl_ids_in_range": [_vp, _i64, _i64, _vp, _vp],
     "ezl_embed_gather": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
     "ezl_embed_scatter_add": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
     "ezl_transpose01": [_vp, _vp, _i64, _i64, _i64, _vp],

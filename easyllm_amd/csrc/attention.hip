@@ -48,13 +48,19 @@ __device__ __forceinline__ int64_t tok_off(int n, int s_len, int64_t ss, int64_t
     return (int64_t)b * sb + (int64_t)(n - b * s_len) * ss;
 }
 
-// block id -> (document, block inside the document); false if the id is beyond the last block.
-// A document is cut at batch-row boundaries (the reference's collator never emits one that crosses a
-// row: it appends every row's length to that row's boundaries), so inside a document token i lives at
-// tok_off(doc_start) + i * seq_stride and no per-token division is needed.
-// The whole workgroup searches together (every thread must call this, before any other use of LDS): thread t counts the
-// blocks of documents t, t + blockDim.x, ..., a prefix sum over the workgroup locates the document that holds block
-// `bid`, and its thread publishes the answer -- ndocs / blockDim.x steps instead of a scalar walk over all documents.
+// Work list of the three kernels.  A document is cut at batch-row boundaries (the reference's collator never emits one
+// that crosses a row: it appends every row's length to that row's boundaries), so inside a piece token i lives at
+// tok_off(piece_start) + i * seq_stride and no per-token division is needed.  A piece of n tokens has ceil(n / 128) blocks;
+// block j of a piece (queries, or keys counted from the piece's END for the dK/dV kernel) walks j + 1 blocks of the other
+// operand, so its running time grows with j.
+//
+// Blocks are handed out longest first over ALL pieces and heads (rank 0 = the largest j anywhere): the hardware starts
+// workgroups in the order of their ids, and with the long blocks of some head started late -- as happens when ids run head
+// by head -- the last of them finish long after everything else (98 instead of 66 block-times for 4 heads x 32 blocks on
+// the 64 slots of an XCD).  rank -> (piece, j): level j holds the pieces with more than j blocks, levels are laid out from
+// the highest down; the level is found by bisection on count(j) = number of blocks with index >= j, the piece inside the
+// level by a prefix sum, both computed by the whole workgroup (every thread must call this, before any other use of LDS).
+// Dense batches (no cu_seqlens) have a closed form.
 __device__ __forceinline__ int doc_bounds(const int* __restrict__ cu, int d, int s_len, int T, int& e) {
     int a = cu ? cu[d] : d * s_len;
     e = cu ? cu[d + 1] : (d + 1) * s_len;
@@ -63,81 +69,136 @@ __device__ __forceinline__ int doc_bounds(const int* __restrict__ cu, int d, int
     return a;
 }
 
-__device__ __forceinline__ bool find_block(const int* __restrict__ cu, int ndocs, int s_len, int T, int bid, int blk_rows,
+struct BlockSearch {
+    int* s_wave;  // [16]
+    int tid, nthr, lane, wv, nwaves;
+    // sum over the workgroup; uniform result
+    __device__ __forceinline__ int reduce(int v) const {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+        __syncthreads();  // s_wave of the previous reduction has been read
+        if (lane == 0) s_wave[wv] = v;
+        __syncthreads();
+        int t = 0;
+        for (int i = 0; i < nwaves; ++i) t += s_wave[i];
+        return t;
+    }
+};
+
+__device__ __forceinline__ bool find_block(const int* __restrict__ cu, int ndocs, int s_len, int T, int rank, int blk_rows,
                                            int& doc_start, int& doc_len, int& blk) {
+    const int nb_row = (s_len + blk_rows - 1) / blk_rows;
+    if (!cu) {  // every piece is a whole batch row: level j holds all ndocs rows
+        if (rank >= ndocs * nb_row) return false;
+        blk = nb_row - 1 - rank / ndocs;
+        doc_start = (rank % ndocs) * s_len;
+        doc_len = s_len;
+        return true;
+    }
     __shared__ int s_wave[16];
     __shared__ int s_found[4];
-    const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63, wv = tid >> 6, nwaves = nthr >> 6;
-    if (tid == 0) s_found[0] = 0;
-    int base = 0;
-    for (int d0 = 0; d0 < ndocs; d0 += nthr) {
-        const int d = d0 + tid;
-        int nb = 0, a = 0, e = 0;
-        if (d < ndocs) {
-            a = doc_bounds(cu, d, s_len, T, e);
-            for (int x = a; x < e;) {  // one pass unless the document crosses a batch row
-                const int row_end = (x / s_len + 1) * s_len;
-                const int e1 = e < row_end ? e : row_end;
-                nb += (e1 - x + blk_rows - 1) / blk_rows;
-                x = e1;
-            }
-        }
-        int incl = nb;
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const int v = __shfl_up(incl, o, 64);
-            if (lane >= o) incl += v;
-        }
-        __syncthreads();  // s_wave of the previous round has been read
-        if (lane == 63) s_wave[wv] = incl;
-        __syncthreads();
-        int before = 0, total = 0;
-        for (int i = 0; i < nwaves; ++i) {
-            const int v = s_wave[i];
-            before += i < wv ? v : 0;
-            total += v;
-        }
-        const int lo = base + before + incl - nb;  // first block id of this thread's document
-        if (nb > 0 && bid >= lo && bid < lo + nb) {
-            int rel = bid - lo;
+    BlockSearch bs;
+    bs.s_wave = s_wave;
+    bs.tid = threadIdx.x; bs.nthr = blockDim.x; bs.lane = bs.tid & 63; bs.wv = bs.tid >> 6; bs.nwaves = bs.nthr >> 6;
+    // blocks with index >= j over this thread's documents (pieces enumerated on the fly; one piece unless a document
+    // crosses a batch row)
+    auto count_ge = [&](int j) {
+        int c = 0;
+        for (int d = bs.tid; d < ndocs; d += bs.nthr) {
+            int e;
+            const int a = doc_bounds(cu, d, s_len, T, e);
             for (int x = a; x < e;) {
                 const int row_end = (x / s_len + 1) * s_len;
                 const int e1 = e < row_end ? e : row_end;
-                const int n1 = (e1 - x + blk_rows - 1) / blk_rows;
-                if (rel < n1) {
-                    s_found[1] = x;
-                    s_found[2] = e1 - x;
-                    s_found[3] = rel;
-                    s_found[0] = 1;
-                    break;
+                const int nb = (e1 - x + blk_rows - 1) / blk_rows;
+                c += nb > j ? nb - j : 0;
+                x = e1;
+            }
+        }
+        return bs.reduce(c);
+    };
+    if (rank >= count_ge(0)) return false;
+    int lo = 0, hi = nb_row, c_hi = 0;  // count(lo) > rank >= count(hi)
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        const int c = count_ge(mid);
+        if (c > rank) lo = mid;
+        else { hi = mid; c_hi = c; }
+    }
+    const int j = lo;
+    const int want = rank - c_hi;  // the want-th piece (in document order) that has more than j blocks
+    if (bs.tid == 0) s_found[0] = 0;
+    int base = 0;
+    for (int d0 = 0; d0 < ndocs; d0 += bs.nthr) {
+        const int d = d0 + bs.tid;
+        int mine = 0, a = 0, e = 0;
+        if (d < ndocs) {
+            a = doc_bounds(cu, d, s_len, T, e);
+            for (int x = a; x < e;) {
+                const int row_end = (x / s_len + 1) * s_len;
+                const int e1 = e < row_end ? e : row_end;
+                mine += (e1 - x + blk_rows - 1) / blk_rows > j;
+                x = e1;
+            }
+        }
+        int incl = mine;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(incl, o, 64);
+            if (bs.lane >= o) incl += v;
+        }
+        __syncthreads();
+        if (bs.lane == 63) s_wave[bs.wv] = incl;
+        __syncthreads();
+        int before = 0, total = 0;
+        for (int i = 0; i < bs.nwaves; ++i) {
+            const int v = s_wave[i];
+            before += i < bs.wv ? v : 0;
+            total += v;
+        }
+        const int first = base + before + incl - mine;  // rank inside the level of this thread's first qualifying piece
+        if (mine > 0 && want >= first && want < first + mine) {
+            int rel = want - first;
+            for (int x = a; x < e;) {
+                const int row_end = (x / s_len + 1) * s_len;
+                const int e1 = e < row_end ? e : row_end;
+                if ((e1 - x + blk_rows - 1) / blk_rows > j) {
+                    if (rel == 0) {
+                        s_found[1] = x;
+                        s_found[2] = e1 - x;
+                        s_found[0] = 1;
+                        break;
+                    }
+                    --rel;
                 }
-                rel -= n1;
                 x = e1;
             }
         }
         base += total;
-        if (bid < base) break;  // uniform: the block lies in this round's documents
+        if (want < base) break;  // uniform
     }
     __syncthreads();
     if (!s_found[0]) return false;
     doc_start = __builtin_amdgcn_readfirstlane(s_found[1]);
     doc_len = __builtin_amdgcn_readfirstlane(s_found[2]);
-    blk = __builtin_amdgcn_readfirstlane(s_found[3]);
+    blk = j;
     return true;
 }
 
 // The hardware deals consecutive workgroups (x fastest, then y) round-robin to the 8 XCDs, each with an L2 of its own.
 // With the plain (block, head) numbering every XCD would touch the K / V rows of every head and its L2 would keep missing;
-// renumbered, an XCD gets whole heads, a few at a time.  by: head, bx: block index inside the head's token blocks.
-__device__ __forceinline__ void xcd_head_blocks(int nheads, int& bx, int& by) {
-    bx = blockIdx.x;
-    by = blockIdx.y;
+// renumbered, an XCD owns nheads / 8 heads, and inside an XCD the ids run over ranks (longest blocks first, see above) with
+// the XCD's heads innermost: blocks of equal length of all its heads start together and walk the keys in step.
+// by: head, rank: position in the longest-first work list of one head.
+__device__ __forceinline__ void xcd_head_blocks(int nheads, int& rank, int& by) {
+    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
     if ((nheads & 7) == 0) {
-        const int gx = gridDim.x;
-        const int lin = blockIdx.y * gx + blockIdx.x;
-        const int idx = lin >> 3;
-        by = (lin & 7) * (nheads >> 3) + idx / gx;
-        bx = idx % gx;
+        const int hpx = nheads >> 3, idx = lin >> 3;
+        by = (lin & 7) * hpx + idx % hpx;
+        rank = idx / hpx;
+    } else {
+        by = lin % nheads;
+        rank = lin / nheads;
     }
 }
 
@@ -234,8 +295,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
     int doc_start, doc_len, qb;
     int bx, by;
     xcd_head_blocks(p.nq, bx, by);
-    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;
-    qb = (doc_len + 127) / 128 - 1 - qb;  // longest rows first
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;  // bx = rank: longest rows first
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hq = by, hk = hq / (p.nq / p.nk);
     const int q0 = qb * 128, qw0 = q0 + wave * 32;
@@ -438,6 +498,7 @@ __global__ __launch_bounds__(kDkdvThreads) void attn_bwd_dkdv_kernel(AttnParams 
     int bx, by;
     xcd_head_blocks(p.nk, bx, by);
     if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, kbk)) return;
+    kbk = (doc_len + 127) / 128 - 1 - kbk;  // rank 0 = most blocks of queries to walk = the piece's first keys
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kg = wave & 3, half = wave >> 2;
     const int hk = by, group = p.nq / p.nk;
@@ -637,8 +698,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
     int doc_start, doc_len, qb;
     int bx, by;
     xcd_head_blocks(p.nq, bx, by);
-    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;
-    qb = (doc_len + 127) / 128 - 1 - qb;
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;  // bx = rank: longest rows first
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hq = by, hk = hq / (p.nq / p.nk);
     const int q0 = qb * 128, qw0 = q0 + wave * 32;

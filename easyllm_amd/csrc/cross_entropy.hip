@@ -313,7 +313,7 @@ __global__ __launch_bounds__(kWideBlock) void ce_fused_wide_kernel(const bf16_t*
     auto fetch_reg = [&](const bf16_t* src, int j) {  // register vector j = row vector (kWideLds + j) * 1024 + tid
         const int i = tid + (kWideLds + j) * kWideBlock;
         if (i < v8) {
-            raw[j] = ld_bf16x8(src + (int64_t)i * 8);
+            raw[j] = ld_bf16x8_nt(src + (int64_t)i * 8);
         } else {
 #pragma unroll
             for (int k = 0; k < 8; ++k) raw[j][k] = (bf16_t)(-INFINITY);
@@ -359,8 +359,7 @@ __global__ __launch_bounds__(kWideBlock) void ce_fused_wide_kernel(const bf16_t*
         }
         const int64_t t = labels[r];
         const bool masked = t < 0 || t >= vend;
-        // the target logit straight from memory (the row is being read anyway): the passes below stay free of per-vector
-        // target tests, and the one-hot term is applied by a single-element fix-up after the gradient pass
+        // the target logit straight from memory (the row is being read anyway): the first two passes stay free of target tests
         const float xt = masked ? 0.f : (float)logits[r * V + t];
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the row is on chip (LDS part included)
         asm volatile("" ::: "memory");           // ... and the compiler may not reuse LDS values read before this point
@@ -418,17 +417,24 @@ __global__ __launch_bounds__(kWideBlock) void ce_fused_wide_kernel(const bf16_t*
         // the block reduction and spill them.
         float mb2 = mb;
         asm volatile("" : "+v"(mb2));
-        auto grad_of = [&](const bf16x8 v) {
+        // one-hot term: the vector that holds the target column belongs to chunk tj (uniform over the block: a scalar test
+        // per chunk), and inside it to thread towner, element tsub
+        const int tj = masked ? -1 : (int)(t >> 3) / kWideBlock, towner = (int)(t >> 3) % kWideBlock, tsub = (int)(t & 7);
+        auto grad_of = [&](const bf16x8 v, bool holds_target) {
             float g[8];
             unpack8(v, g);
 #pragma unroll
             for (int k = 0; k < 8; ++k) g[k] = __builtin_amdgcn_exp2f(g[k] * kLog2e - mb2) * ps;
+            if (holds_target) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) g[k] -= (k == tsub && tid == towner) ? scale : 0.f;
+            }
             return pack8(g);
         };
 #pragma unroll
         for (int j = 0; j < kWideLds; ++j) {
             const int i = tid + j * kWideBlock;
-            st_bf16x8(grow + (int64_t)i * 8, grad_of(lds_vec(j)));
+            st_bf16x8_nt(grow + (int64_t)i * 8, grad_of(lds_vec(j), j == tj));
             // the LDS read above has returned (its value was used): the slot may be refilled with the next row
             fetch_lds(next, j);
         }
@@ -436,14 +442,10 @@ __global__ __launch_bounds__(kWideBlock) void ce_fused_wide_kernel(const bf16_t*
         for (int j = 0; j < NR; ++j) {
             const int i = tid + (kWideLds + j) * kWideBlock;
             asm volatile("" : "+v"(raw[j]));
-            const bf16x8 gv = grad_of(raw[j]);
-            if (i < v8) st_bf16x8(grow + (int64_t)i * 8, gv);
+            const bf16x8 gv = grad_of(raw[j], kWideLds + j == tj);
+            if (i < v8) st_bf16x8_nt(grow + (int64_t)i * 8, gv);
             fetch_reg(next, j);  // this vector's registers are free: start the next row's fetch behind the store
         }
-        // one-hot term: the thread that stored the vector holding the target column rewrites that one element (stores of
-        // one thread to one address keep their order)
-        if (!masked && tid == (int)((t >> 3) & (kWideBlock - 1)))
-            grow[t] = (bf16_t)(__builtin_amdgcn_exp2f(xt * kLog2e - mb2) * ps - scale);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // no LDS write of this block may still be in flight when it ends
 }

@@ -26,11 +26,11 @@ __global__ __launch_bounds__(kBlock) void swiglu_fwd_kernel(const bf16_t* __rest
                                                             bf16_t* __restrict__ out, int64_t n8) {
     for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += (int64_t)gridDim.x * kBlock) {
         float g[8], u[8], o[8];
-        unpack8(ld_bf16x8(gate + i * 8), g);
-        unpack8(ld_bf16x8(up + i * 8), u);
+        unpack8(ld_bf16x8_nt(gate + i * 8), g);
+        unpack8(ld_bf16x8_nt(up + i * 8), u);
 #pragma unroll
         for (int k = 0; k < 8; ++k) o[k] = g[k] * sigmoidf_fast(g[k]) * u[k];
-        st_bf16x8(out + i * 8, pack8(o));
+        st_bf16x8_nt(out + i * 8, pack8(o));
     }
 }
 
@@ -40,17 +40,17 @@ __global__ __launch_bounds__(kBlock) void swiglu_bwd_kernel(const bf16_t* __rest
                                                             bf16_t* __restrict__ dup, int64_t n8) {
     for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += (int64_t)gridDim.x * kBlock) {
         float g[8], u[8], d[8], dg[8], du[8];
-        unpack8(ld_bf16x8(gate + i * 8), g);
-        unpack8(ld_bf16x8(up + i * 8), u);
-        unpack8(ld_bf16x8(dout + i * 8), d);
+        unpack8(ld_bf16x8_nt(gate + i * 8), g);
+        unpack8(ld_bf16x8_nt(up + i * 8), u);
+        unpack8(ld_bf16x8_nt(dout + i * 8), d);
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             const float s = sigmoidf_fast(g[k]);
             dg[k] = d[k] * u[k] * s * (1.0f + g[k] * (1.0f - s));
             du[k] = d[k] * g[k] * s;
         }
-        st_bf16x8(dgate + i * 8, pack8(dg));
-        st_bf16x8(dup + i * 8, pack8(du));
+        st_bf16x8_nt(dgate + i * 8, pack8(dg));
+        st_bf16x8_nt(dup + i * 8, pack8(du));
     }
 }
 
@@ -74,28 +74,38 @@ __global__ __launch_bounds__(kBlock) void rope_table_kernel(const float* __restr
 
 // x [rows = s*b (s-major), nheads, d] with a row stride; one work item = 8 low-half + 8 high-half
 // elements of one head.  out1 = x1*c - sign*x2*s ; out2 = x2*c + sign*x1*s  (sign = -1: backward).
-__global__ __launch_bounds__(kBlock) void rope_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ out,
-                                                      const float* __restrict__ cosb, const float* __restrict__ sinb,
-                                                      const int64_t* __restrict__ position_ids, int64_t rows, int s,
-                                                      int b, int nheads, int d, int64_t in_stride, int64_t out_stride,
-                                                      int64_t npos, float sign) {
+// Two tensors that share their rows (q and k of one layer: nheads0 + nheads1 heads per row) go through one launch; the
+// second is absent when nheads1 == 0.
+struct RopeSide {
+    const bf16_t* x;
+    bf16_t* out;
+    int64_t in_stride, out_stride;
+};
+
+__global__ __launch_bounds__(kBlock) void rope_kernel(RopeSide a, RopeSide b2, const float* __restrict__ cosb,
+                                                      const float* __restrict__ sinb, const int64_t* __restrict__ position_ids,
+                                                      int64_t rows, int s, int b, int nheads0, int nheads1, int d, int64_t npos,
+                                                      float sign) {
     const int half = d >> 1;
     const int per_head = half >> 3;
+    const int nheads = nheads0 + nheads1;
     const int64_t items = rows * nheads * per_head;
     for (int64_t it = (int64_t)blockIdx.x * kBlock + threadIdx.x; it < items; it += (int64_t)gridDim.x * kBlock) {
         const int j8 = (int)(it % per_head);
         const int64_t rh = it / per_head;
-        const int head = (int)(rh % nheads);
+        int head = (int)(rh % nheads);
         const int64_t row = rh / nheads;
         const int si = (int)(row / b), bi = (int)(row % b);
         int64_t pos = position_ids ? position_ids[(int64_t)bi * s + si] : si;
         pos = pos < 0 ? 0 : (pos >= npos ? npos - 1 : pos);
         const float* cp = cosb + pos * half + j8 * 8;
         const float* sp = sinb + pos * half + j8 * 8;
-        const bf16_t* xi = x + row * in_stride + (int64_t)head * d + j8 * 8;
-        bf16_t* xo = out + row * out_stride + (int64_t)head * d + j8 * 8;
-        float a[8], c[8], o1[8], o2[8];
-        unpack8(ld_bf16x8(xi), a);
+        const bool second = head >= nheads0;
+        head -= second ? nheads0 : 0;
+        const bf16_t* xi = (second ? b2.x : a.x) + row * (second ? b2.in_stride : a.in_stride) + (int64_t)head * d + j8 * 8;
+        bf16_t* xo = (second ? b2.out : a.out) + row * (second ? b2.out_stride : a.out_stride) + (int64_t)head * d + j8 * 8;
+        float av[8], c[8], o1[8], o2[8];
+        unpack8(ld_bf16x8(xi), av);
         unpack8(ld_bf16x8(xi + half), c);
         const f32x4 c0 = *reinterpret_cast<const f32x4*>(cp), c1 = *reinterpret_cast<const f32x4*>(cp + 4);
         const f32x4 s0 = *reinterpret_cast<const f32x4*>(sp), s1 = *reinterpret_cast<const f32x4*>(sp + 4);
@@ -103,8 +113,8 @@ __global__ __launch_bounds__(kBlock) void rope_kernel(const bf16_t* __restrict__
         for (int k = 0; k < 8; ++k) {
             const float cs = k < 4 ? c0[k] : c1[k - 4];
             const float sn = sign * (k < 4 ? s0[k] : s1[k - 4]);
-            o1[k] = a[k] * cs - c[k] * sn;
-            o2[k] = c[k] * cs + a[k] * sn;
+            o1[k] = av[k] * cs - c[k] * sn;
+            o2[k] = c[k] * cs + av[k] * sn;
         }
         st_bf16x8(xo, pack8(o1));
         st_bf16x8(xo + half, pack8(o2));
@@ -114,21 +124,41 @@ __global__ __launch_bounds__(kBlock) void rope_kernel(const bf16_t* __restrict__
 // ---------------------------------------------------------------------------------------------
 // Token embedding (base_modules/layers/vocab_parallel_emb.py:106-137, TP=1)
 // ---------------------------------------------------------------------------------------------
+// ORs 1 into *bad_flag if some id >= limit, 2 if some id < 0 (the range test of an index tensor, without a host sync)
+__global__ __launch_bounds__(kBlock) void ids_in_range_kernel(const int64_t* __restrict__ ids, int64_t n, int64_t limit,
+                                                              int* __restrict__ bad_flag) {
+    int bad = 0;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+        const int64_t id = ids[i];
+        bad |= id >= limit ? 1 : (id < 0 ? 2 : 0);
+    }
+    if (bad) atomicOr(bad_flag, bad);
+}
+
 // out[r, :] = W[ids[r], :]; an id outside [0, V) raises the flag and yields a zero row.
+// One wave per row; a lane's loads (up to 4 vectors of 8 at a time) are all in flight before its first store.
 __global__ __launch_bounds__(kBlock) void embed_gather_kernel(const int64_t* __restrict__ ids, const bf16_t* __restrict__ W,
                                                               bf16_t* __restrict__ out, int64_t rows, int h, int64_t V,
                                                               int* __restrict__ bad_flag) {
     const int h8 = h >> 3;
-    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int64_t r = (int64_t)blockIdx.x * 4 + wave; r < rows; r += (int64_t)gridDim.x * 4) {
         const int64_t id = ids[r];
         const bool ok = id >= 0 && id < V;
-        if (!ok && threadIdx.x == 0) atomicOr(bad_flag, id >= V ? 1 : 2);
-        for (int c = threadIdx.x; c < h8; c += kBlock) {
-            bf16x8 v;
+        if (!ok && lane == 0) atomicOr(bad_flag, id >= V ? 1 : 2);
+        const bf16_t* src = W + (ok ? id : 0) * h;
+        bf16_t* dst = out + r * h;
+        for (int c0 = lane; c0 < h8; c0 += 256) {
+            bf16x8 v[4];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] = (bf16_t)0.0f;
-            if (ok) v = ld_bf16x8(W + id * h + c * 8);
-            st_bf16x8(out + r * h + c * 8, v);
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) v[u][k] = (bf16_t)0.0f;
+                if (ok && c0 + u * 64 < h8) v[u] = ld_bf16x8(src + (c0 + u * 64) * 8);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (c0 + u * 64 < h8) st_bf16x8(dst + (c0 + u * 64) * 8, v[u]);
         }
     }
 }
@@ -453,24 +483,54 @@ extern "C" int ezl_rope_table(const void* inv_freq, void* cos_out, void* sin_out
     return EZL_OK;
 }
 
+namespace {
+int rope_launch(const char* name, const void* x0, void* out0, int64_t nh0, int64_t is0, int64_t os0, const void* x1, void* out1,
+                int64_t nh1, int64_t is1, int64_t os1, const void* cos_table, const void* sin_table, const void* position_ids,
+                int64_t s, int64_t b, int64_t d, int64_t npos, int backward, void* stream) {
+    EZL_REQUIRE(s >= 0 && b > 0 && nh0 > 0 && nh1 >= 0 && d > 0 && d % 16 == 0, EZL_EUNSUPPORTED,
+                "%s: head dim must be a multiple of 16 (got %lld)", name, (long long)d);
+    EZL_REQUIRE(is0 % 8 == 0 && os0 % 8 == 0 && is0 >= nh0 * d && os0 >= nh0 * d, EZL_EINVAL, "%s: bad row stride", name);
+    EZL_REQUIRE(nh1 == 0 || (is1 % 8 == 0 && os1 % 8 == 0 && is1 >= nh1 * d && os1 >= nh1 * d), EZL_EINVAL, "%s: bad row stride", name);
+    EZL_REQUIRE(npos >= 1 && (position_ids || npos >= s), EZL_EINVAL, "%s: cos/sin table shorter than the sequence", name);
+    EZL_REQUIRE((s == 0 || (x0 && out0 && (nh1 == 0 || (x1 && out1)))) && cos_table && sin_table && ezl_aligned16(x0) &&
+                    ezl_aligned16(out0) && ezl_aligned16(x1) && ezl_aligned16(out1) && ezl_aligned16(cos_table) &&
+                    ezl_aligned16(sin_table),
+                EZL_EINVAL, "%s: null or misaligned pointer", name);
+    EZL_REQUIRE(s < (1LL << 31) && b < (1LL << 31) && nh0 + nh1 < (1LL << 24), EZL_EUNSUPPORTED, "%s: shape too large", name);
+    if (s == 0) return EZL_OK;
+    const int64_t items = s * b * (nh0 + nh1) * (d / 16);
+    const RopeSide a = {(const bf16_t*)x0, (bf16_t*)out0, is0, os0};
+    const RopeSide c = {(const bf16_t*)x1, (bf16_t*)out1, is1, os1};
+    hipLaunchKernelGGL(rope_kernel, dim3(grid_for(items, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, a, c,
+                       (const float*)cos_table, (const float*)sin_table, (const int64_t*)position_ids, s * b, (int)s, (int)b,
+                       (int)nh0, (int)nh1, (int)d, npos, backward ? -1.0f : 1.0f);
+    EZL_LAUNCH_CHECK(name);
+    return EZL_OK;
+}
+}  // namespace
+
 extern "C" int ezl_rope_apply(const void* x, void* out, const void* cos_table, const void* sin_table,
                               const void* position_ids, int64_t s, int64_t b, int64_t nheads, int64_t d,
                               int64_t in_row_stride, int64_t out_row_stride, int64_t npos, int backward, void* stream) {
-    EZL_REQUIRE(s >= 0 && b > 0 && nheads > 0 && d > 0 && d % 16 == 0, EZL_EUNSUPPORTED,
-                "ezl_rope_apply: head dim must be a multiple of 16 (got %lld)", (long long)d);
-    EZL_REQUIRE(in_row_stride % 8 == 0 && out_row_stride % 8 == 0 && in_row_stride >= nheads * d && out_row_stride >= nheads * d,
-                EZL_EINVAL, "ezl_rope_apply: bad row stride");
-    EZL_REQUIRE(npos >= 1 && (position_ids || npos >= s), EZL_EINVAL, "ezl_rope_apply: cos/sin table shorter than the sequence");
-    EZL_REQUIRE((s == 0 || (x && out)) && cos_table && sin_table && ezl_aligned16(x) && ezl_aligned16(out) &&
-                    ezl_aligned16(cos_table) && ezl_aligned16(sin_table),
-                EZL_EINVAL, "ezl_rope_apply: null or misaligned pointer");
-    EZL_REQUIRE(s < (1LL << 31) && b < (1LL << 31), EZL_EUNSUPPORTED, "ezl_rope_apply: shape too large");
-    if (s == 0) return EZL_OK;
-    const int64_t items = s * b * nheads * (d / 16);
-    hipLaunchKernelGGL(rope_kernel, dim3(grid_for(items, kBlock)), dim3(kBlock), 0, (hipStream_t)stream, (const bf16_t*)x,
-                       (bf16_t*)out, (const float*)cos_table, (const float*)sin_table, (const int64_t*)position_ids, s * b,
-                       (int)s, (int)b, (int)nheads, (int)d, in_row_stride, out_row_stride, npos, backward ? -1.0f : 1.0f);
-    EZL_LAUNCH_CHECK("ezl_rope_apply");
+    return rope_launch("ezl_rope_apply", x, out, nheads, in_row_stride, out_row_stride, nullptr, nullptr, 0, 0, 0, cos_table,
+                       sin_table, position_ids, s, b, d, npos, backward, stream);
+}
+
+extern "C" int ezl_rope_apply_pair(const void* q, void* q_out, int64_t nq, int64_t q_in_stride, int64_t q_out_stride,
+                                   const void* k, void* k_out, int64_t nk, int64_t k_in_stride, int64_t k_out_stride,
+                                   const void* cos_table, const void* sin_table, const void* position_ids, int64_t s, int64_t b,
+                                   int64_t d, int64_t npos, int backward, void* stream) {
+    EZL_REQUIRE(nk > 0, EZL_EINVAL, "ezl_rope_apply_pair: the second tensor needs at least one head");
+    return rope_launch("ezl_rope_apply_pair", q, q_out, nq, q_in_stride, q_out_stride, k, k_out, nk, k_in_stride, k_out_stride,
+                       cos_table, sin_table, position_ids, s, b, d, npos, backward, stream);
+}
+
+extern "C" int ezl_ids_in_range(const void* ids, int64_t n, int64_t limit, void* bad_flag, void* stream) {
+    EZL_REQUIRE(n >= 0 && bad_flag && (n == 0 || ids), EZL_EINVAL, "ezl_ids_in_range: null pointer");
+    if (n == 0) return EZL_OK;
+    hipLaunchKernelGGL(ids_in_range_kernel, dim3(grid_for(n, kBlock, 256)), dim3(kBlock), 0, (hipStream_t)stream, (const int64_t*)ids,
+                       n, limit, (int*)bad_flag);
+    EZL_LAUNCH_CHECK("ezl_ids_in_range");
     return EZL_OK;
 }
 
@@ -481,7 +541,7 @@ extern "C" int ezl_embed_gather(const void* ids, const void* weight, void* out, 
     EZL_REQUIRE(bad_flag && (rows == 0 || (ids && weight && out)) && ezl_aligned16(weight) && ezl_aligned16(out), EZL_EINVAL,
                 "ezl_embed_gather: null or misaligned pointer");
     if (rows == 0) return EZL_OK;
-    hipLaunchKernelGGL(embed_gather_kernel, dim3(grid_for(rows, 1)), dim3(kBlock), 0, (hipStream_t)stream, (const int64_t*)ids,
+    hipLaunchKernelGGL(embed_gather_kernel, dim3(grid_for((rows + 3) / 4, 1)), dim3(kBlock), 0, (hipStream_t)stream, (const int64_t*)ids,
                        (const bf16_t*)weight, (bf16_t*)out, rows, (int)h, vocab, (int*)bad_flag);
     EZL_LAUNCH_CHECK("ezl_embed_gather");
     return EZL_OK;

@@ -5,10 +5,9 @@
 // of llama/transformer.py:786 fused in front (sum rounded to bf16 first, as the reference's bf16
 // tensor add does).
 //
-// Layout: rows of h bf16, h % 8 == 0, h <= 8192.  A row is owned by TPR = min(256, h/8 rounded up
-// to a wave) threads, each holding NCHUNK 128-bit column groups in registers, so a row is read
-// from HBM exactly once.  Row sums reduce with wave shuffles, then across the (<= 4) waves of the
-// row slot through a double-buffered LDS cell (one barrier per row).
+// Layout: rows of h bf16, h % 8 == 0, h <= 8192.  A row is held in registers (read from HBM exactly once) by
+// TPR = min(256, h/8 rounded up to a wave) threads whose row sums meet through a double-buffered LDS cell (forward;
+// backward for h > 4096, one barrier per row), or by one wave (backward for h <= 4096).
 #include "common.h"
 
 #include <mutex>
@@ -194,6 +193,91 @@ __global__ __launch_bounds__(1024) void rmsnorm_bwd_kernel(const bf16_t* __restr
     for (int j = threadIdx.x; j < h; j += 1024) dw_partial[(size_t)blockIdx.x * h + j] = fold[j];
 }
 
+// ---- backward with one wave per row (h <= 4096) ----------------------------------------------------------------
+// A row is owned by ONE wave: lane l holds the 8 columns (c * 64 + l) * 8 .. + 7 of chunk c, so every chunk is one
+// coalesced 1 KiB access, the row sums need wave shuffles only and there is no barrier inside the row loop: the waves
+// of a CU run out of step and keep HBM busy while others compute.  Loads and stores carry the streaming hint (in the
+// step: 42 -> 34 us); the forward kernel keeps the block-per-row form and plain accesses, which measured faster there
+// (its input was written by the kernel before it and its output is read by the one after, 33 MB each).
+// Backward, 8 waves per block: each wave keeps the dw partial of its lanes' columns over all rows it visits; at the end the
+// 8 waves of a block are folded through LDS in a fixed order and one partial row per block goes to HBM.
+template <int NCHUNK, bool HAS_DRES>
+__global__ __launch_bounds__(512) void rmsnorm_bwd_wave_kernel(const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
+                                                               const bf16_t* __restrict__ w, const float* __restrict__ rstd,
+                                                               const bf16_t* __restrict__ dres, bf16_t* __restrict__ dx,
+                                                               float* __restrict__ dw_partial, int T, int h) {
+    extern __shared__ float fold[];  // h floats
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    bf16x8 wr[NCHUNK];
+    float dwacc[NCHUNK][8];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+        const int col = (c * 64 + lane) * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { dwacc[c][i] = 0.f; wr[c][i] = (bf16_t)0.0f; }
+        if (col < h) wr[c] = ld_bf16x8(w + col);
+    }
+    const float inv_h = 1.0f / (float)h;
+    for (int row = blockIdx.x * 8 + wave; row < T; row += gridDim.x * 8) {
+        const size_t base = (size_t)row * h;
+        const float rs = rstd[row];
+        bf16x8 xr[NCHUNK], dyr[NCHUNK], drr[NCHUNK];
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            const int col = (c * 64 + lane) * 8;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { xr[c][i] = (bf16_t)0.0f; dyr[c][i] = (bf16_t)0.0f; }
+            if (col < h) {
+                xr[c] = ld_bf16x8_nt(x + base + col);
+                dyr[c] = ld_bf16x8_nt(dy + base + col);
+                if (HAS_DRES) drr[c] = ld_bf16x8_nt(dres + base + col);
+            }
+        }
+        float dot = 0.f;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dot += (float)dyr[c][i] * (float)wr[c][i] * ((float)xr[c][i] * rs);
+        dot = wave_sum(dot);
+        const float cmean = dot * inv_h;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            const int col = (c * 64 + lane) * 8;
+            // opaque to the compiler: the fp32 copies made for the dot product must not be kept alive (they would not fit)
+            asm volatile("" : "+v"(xr[c]), "+v"(dyr[c]));
+            if (col < h) {
+                float o[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float xhat = (float)xr[c][i] * rs;
+                    const float dyv = (float)dyr[c][i];
+                    o[i] = rs * (dyv * (float)wr[c][i] - xhat * cmean);
+                    if (HAS_DRES) o[i] += (float)drr[c][i];
+                    dwacc[c][i] += dyv * xhat;
+                }
+                st_bf16x8_nt(dx + base + col, pack8(o));
+            }
+        }
+    }
+    for (int s = 0; s < 8; ++s) {  // wave 0 stores, the others add in turn: a fixed order
+        if (wave == s) {
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c) {
+                const int col = (c * 64 + lane) * 8;
+                if (col < h) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        if (s == 0) fold[col + i] = dwacc[c][i];
+                        else fold[col + i] += dwacc[c][i];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    for (int j = threadIdx.x; j < h; j += 512) dw_partial[(size_t)blockIdx.x * h + j] = fold[j];
+}
+
 int tpr_for(int h) {
     int t = (h / 8 + 63) / 64 * 64;
     return t < 64 ? 64 : (t > 256 ? 256 : t);
@@ -255,23 +339,45 @@ int rmsnorm_bwd_check(const char* name, const void* dy, const void* x, const voi
 // both entry points: `partials` holds one fp32 row of h per block (at most 256 blocks), every used row fully written
 int rmsnorm_bwd_launch(const void* dy, const void* x, const void* weight, const void* rstd, const void* dresidual, void* dx,
                        void* dw_bf16, void* dw_f32, int accumulate, float* partials, int64_t rows, int64_t h, hipStream_t st) {
-    const int tpr = tpr_for((int)h);
-    const int nchunk = ((int)h + tpr * 8 - 1) / (tpr * 8);
-    const int rpb = 1024 / tpr;
-    int64_t grid = (rows + rpb - 1) / rpb;
-    if (grid > 256) grid = 256;
-    if (grid < 1) grid = 1;  // rows == 0 still produces a zero dw
     const size_t smem = (size_t)h * sizeof(float);
+    int64_t grid;
+    if (h <= 4096) {  // one wave per row, 8 rows per block
+        const int nchunk = ((int)h + 511) / 512;
+        grid = (rows + 7) / 8;
+        if (grid > 256) grid = 256;
+        if (grid < 1) grid = 1;  // rows == 0 still produces a zero dw
+#define LAUNCH(NC, DR)                                                                                                    \
+    hipLaunchKernelGGL((rmsnorm_bwd_wave_kernel<NC, DR>), dim3((unsigned)grid), dim3(512), smem, st, (const bf16_t*)dy,    \
+                       (const bf16_t*)x, (const bf16_t*)weight, (const float*)rstd, (const bf16_t*)dresidual, (bf16_t*)dx, \
+                       partials, (int)rows, (int)h)
+#define LAUNCH_NC(DR)                                  \
+    do {                                               \
+        if (nchunk <= 1) LAUNCH(1, DR);                \
+        else if (nchunk <= 2) LAUNCH(2, DR);           \
+        else if (nchunk <= 4) LAUNCH(4, DR);           \
+        else LAUNCH(8, DR);                            \
+    } while (0)
+        if (dresidual) LAUNCH_NC(true); else LAUNCH_NC(false);
+#undef LAUNCH_NC
+#undef LAUNCH
+    } else {  // wider rows: 256 threads per row, row sums across waves through LDS
+        const int tpr = tpr_for((int)h);
+        const int nchunk = ((int)h + tpr * 8 - 1) / (tpr * 8);
+        const int rpb = 1024 / tpr;
+        grid = (rows + rpb - 1) / rpb;
+        if (grid > 256) grid = 256;
+        if (grid < 1) grid = 1;
 #define LAUNCH(NC, DR)                                                                                            \
     hipLaunchKernelGGL((rmsnorm_bwd_kernel<NC, DR>), dim3((unsigned)grid), dim3(1024), smem, st, (const bf16_t*)dy, \
                        (const bf16_t*)x, (const bf16_t*)weight, (const float*)rstd, (const bf16_t*)dresidual,     \
                        (bf16_t*)dx, partials, (int)rows, (int)h, tpr)
-    if (dresidual) {
-        if (nchunk == 1) LAUNCH(1, true); else if (nchunk == 2) LAUNCH(2, true); else LAUNCH(4, true);
-    } else {
-        if (nchunk == 1) LAUNCH(1, false); else if (nchunk == 2) LAUNCH(2, false); else LAUNCH(4, false);
-    }
+        if (dresidual) {
+            if (nchunk == 1) LAUNCH(1, true); else if (nchunk == 2) LAUNCH(2, true); else LAUNCH(4, true);
+        } else {
+            if (nchunk == 1) LAUNCH(1, false); else if (nchunk == 2) LAUNCH(2, false); else LAUNCH(4, false);
+        }
 #undef LAUNCH
+    }
     EZL_LAUNCH_CHECK("ezl_rmsnorm_bwd");
     hipLaunchKernelGGL(ezl_colsum_kernel<0>, dim3((unsigned)((h + 63) / 64)), dim3(kColsumThreads), 0, st, (const float*)partials,
                        (int)grid, (int)h, (bf16_t*)dw_bf16, (float*)dw_f32, accumulate);

@@ -234,6 +234,29 @@ def apply_rotary(x, cos, sin, position_ids=None):
     return RotaryFunction.apply(x, cos, sin, position_ids)
 
 
+class RotaryPairFunction(torch.autograd.Function):
+    """(q, k) -> rotated copies in one launch; backward rotates both gradients by the negative angle in one launch."""
+
+    @staticmethod
+    def forward(ctx, q, k, cos, sin, position_ids):
+        ctx.save_for_backward(cos, sin, position_ids)
+        return K.rope_apply_pair(q, k, cos, sin, position_ids)
+
+    @staticmethod
+    def backward(ctx, dq, dk):
+        cos, sin, position_ids = ctx.saved_tensors
+        if dq.stride(3) != 1 or dq.stride(2) != dq.shape[3]:
+            dq = dq.contiguous()
+        if dk.stride(3) != 1 or dk.stride(2) != dk.shape[3]:
+            dk = dk.contiguous()
+        gq, gk = K.rope_apply_pair(dq, dk, cos, sin, position_ids, backward=True)
+        return gq, gk, None, None, None
+
+
+def apply_rotary_pair(q, k, cos, sin, position_ids=None):
+    return RotaryPairFunction.apply(q, k, cos, sin, position_ids)
+
+
 # --------------------------------------------------------------------------------------------
 # attention: llama/transformer.py:83-143
 # --------------------------------------------------------------------------------------------
@@ -319,6 +342,10 @@ class EmbeddingFunction(torch.autograd.Function):
 
 
 def _raise_for_id_flag(bad, ids, num_embeddings):
+    if isinstance(num_embeddings, tuple):  # ("position", table length): the rotary tables' index check
+        if bad:
+            raise IndexError("position id outside the rotary table [0, %d)" % num_embeddings[1])
+        return
     if bad & 1:
         raise ValueError("There is an input id in the input that is greater than the highest possible input id.\n"
                          "Input: {}\nnum_embeddings: {}".format(ids, num_embeddings))
@@ -352,23 +379,34 @@ def flush_input_checks(wait=True):
         _raise_for_id_flag(int(host.item()), ids, n)
 
 
-def embedding(ids, weight):
-    """Row gather; raises ValueError for an id >= vocab like the reference (:107-109)."""
-    out, flag = EmbeddingFunction.apply(ids, weight)
+def _dispatch_flag(flag, ids, limit_tag):
+    """Examines a device flag according to the input-check mode (see set_input_check)."""
     if torch.cuda.is_current_stream_capturing():
-        # inside a graph capture nothing may synchronise: the flag tensor is handed to whoever captures
-        # (runner.GraphedStep), which reads it back after each replay
-        CAPTURED_ID_FLAGS.append((flag, weight.shape[0]))
-        return out
+        CAPTURED_ID_FLAGS.append((flag, limit_tag))
+        return
     if _INPUT_CHECK == "deferred":
         flush_input_checks(wait=False)
         host = torch.empty(1, dtype=torch.int32, pin_memory=True)
         host.copy_(flag, non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
-        _PENDING_CHECKS.append((ev, host, ids, weight.shape[0]))
-        return out
-    _raise_for_id_flag(int(flag.item()), ids, weight.shape[0])
+        _PENDING_CHECKS.append((ev, host, ids, limit_tag))
+        return
+    _raise_for_id_flag(int(flag.item()), ids, limit_tag)
+
+
+def check_position_ids(position_ids, table_len):
+    """IndexError for a position id outside [0, table_len), as indexing the reference's cos / sin tables would give
+    (positional_embeddings.py:109-117); sync or deferred like the token-id check."""
+    _dispatch_flag(K.ids_in_range_flag(position_ids.contiguous(), table_len), position_ids, ("position", int(table_len)))
+
+
+def embedding(ids, weight):
+    """Row gather; raises ValueError for an id >= vocab like the reference (:107-109)."""
+    out, flag = EmbeddingFunction.apply(ids, weight)
+    # inside a graph capture nothing may synchronise: the flag tensor is handed to whoever captures (runner.GraphedStep),
+    # which reads it back after each replay
+    _dispatch_flag(flag, ids, weight.shape[0])
     return out
 
 

@@ -131,6 +131,41 @@ def rope_apply(x, cos, sin, position_ids=None, backward=False, out=None):
     return out
 
 
+def _rope_side(x, out):
+    """(row stride of x, out tensor, row stride of out) for a [s, b, heads, d] tensor with contiguous heads*d."""
+    s, b, nh, d = x.shape
+    _need(x.is_cuda and x.dtype == BF16 and x.dim() == 4, "x must be a bf16 [s, b, heads, d] GPU tensor")
+    _need(x.stride(3) == 1 and x.stride(2) == d and (b == 1 or x.stride(0) == b * x.stride(1)), "rope_apply: unsupported strides")
+    if out is None:
+        out = torch.empty((s, b, nh, d), dtype=BF16, device=x.device)
+    _need(out.stride(3) == 1 and out.stride(2) == d and (b == 1 or out.stride(0) == b * out.stride(1)),
+          "rope_apply: unsupported out strides")
+    return (x.stride(1) if b > 1 else x.stride(0)), out, (out.stride(1) if b > 1 else out.stride(0))
+
+
+def rope_apply_pair(q, k, cos, sin, position_ids=None, backward=False):
+    """Rotates q [s, b, nq, d] and k [s, b, nk, d] in one launch; returns contiguous results."""
+    s, b, nq, d = q.shape
+    _need(k.shape[0] == s and k.shape[1] == b and k.shape[3] == d, "rope_apply_pair: q / k shapes differ")
+    qs, qo, qos = _rope_side(q, None)
+    ks, ko, kos = _rope_side(k, None)
+    if position_ids is not None:
+        _need(position_ids.is_cuda and position_ids.dtype == torch.int64 and position_ids.is_contiguous()
+              and tuple(position_ids.shape) == (b, s), "position_ids must be int64 [b, s]")
+    _need(cos.shape == sin.shape and cos.shape[1] == d // 2 and cos.dtype == torch.float32, "bad cos/sin table")
+    _lib.call("ezl_rope_apply_pair", _p(q), _p(qo), nq, qs, qos, _p(k), _p(ko), k.shape[2], ks, kos, _p(cos), _p(sin),
+              _p(position_ids), s, b, d, cos.shape[0], 1 if backward else 0, _stream())
+    return qo, ko
+
+
+def ids_in_range_flag(ids, limit):
+    """-> int32 [1] GPU flag: bit 0 set if some id >= limit, bit 1 if some id < 0."""
+    _need(ids.is_cuda and ids.dtype == torch.int64 and ids.is_contiguous(), "ids must be contiguous int64 on the GPU")
+    flag = torch.zeros(1, dtype=torch.int32, device=ids.device)
+    _lib.call("ezl_ids_in_range", _p(ids), ids.numel(), int(limit), _p(flag), _stream())
+    return flag
+
+
 # ------------------------------------------------------------------------------------- embedding
 def embed_gather(ids, weight):
     _need(ids.is_cuda and ids.dtype == torch.int64 and ids.is_contiguous(), "ids must be contiguous int64 on the GPU")

@@ -46,4 +46,4 @@ class RotaryEmbedding(torch.nn.Module):
 def apply_rotary_pos_emb(q, k, cos_half, sin_half, position_ids=None):
     """q [s, b, nq, d], k [s, b, nk, d] -> rotated (q, k); position_ids int64 [b, s] or None
     (positions = sequence index), cf. apply_rotary_pos_emb_torch (:105-122)."""
-    return F_.apply_rotary(q, cos_half, sin_half, position_ids), F_.apply_rotary(k, cos_half, sin_half, position_ids)
+    return F_.apply_rotary_pair(q, k, cos_half, sin_half, position_ids)

@@ -2,6 +2,7 @@
 import torch
 
 from . import dist_env
+from . import functional as F_
 from .layers import VocabParallelEmbedding, get_initializer_from_cfg, get_torch_dtype
 
 
@@ -37,6 +38,8 @@ class EmbeddingPipe(Embedding):
         input_ids, position_ids, attention_mask = inputs[0], inputs[1], inputs[2]
         embeddings = super().forward(input_ids, position_ids)
         if len(inputs) == 4:
+            # the layers index their rotary tables (one row per sequence position) with these ids
+            F_.check_position_ids(position_ids, input_ids.shape[1])
             return embeddings, attention_mask, inputs[3], position_ids
         # with a 3-tuple the mask and the position ids are dropped here, as in the reference (:169-172)
         return embeddings

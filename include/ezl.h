@@ -65,6 +65,15 @@ int ezl_rope_table(const void* inv_freq, void* cos_out, void* sin_out, int64_t n
 int ezl_rope_apply(const void* x, void* out, const void* cos_table, const void* sin_table, const void* position_ids, int64_t s,
                    int64_t b, int64_t nheads, int64_t d, int64_t in_row_stride, int64_t out_row_stride, int64_t npos,
                    int backward, void* stream);
+/* range test of the position ids that index the tables (the reference's cos[position_ids], positional_embeddings.py:109-117,
+ * fails on an index past the table): ORs 1 into *bad_flag (device int32) if some id >= limit, 2 if some id < 0.  The apply
+ * kernels themselves clamp. */
+int ezl_ids_in_range(const void* ids_i64, int64_t n, int64_t limit, void* bad_flag, void* stream);
+/* the same rotation of q [.., nq, d] and k [.., nk, d] of one layer (llama/transformer.py:437-448) in one launch */
+int ezl_rope_apply_pair(const void* q, void* q_out, int64_t nq, int64_t q_in_stride, int64_t q_out_stride, const void* k,
+                        void* k_out, int64_t nk, int64_t k_in_stride, int64_t k_out_stride, const void* cos_table,
+                        const void* sin_table, const void* position_ids, int64_t s, int64_t b, int64_t d, int64_t npos,
+                        int backward, void* stream);
 
 /* ---- token embedding: base_modules/layers/vocab_parallel_emb.py:106-137 (F.embedding, TP=1) ----
  * gather: out[r] = weight[ids[r]] (bit-exact row copy); an id outside [0, vocab) ORs 1 (id >= vocab)

@@ -111,6 +111,23 @@ def test_rope(K, gpu_device, s, b, nh, d, use_pos):
     close(qv, ref2, "rope in place, strided", rel=1e-2)
 
 
+def test_rope_pair_equals_two_single_launches(K, gpu_device):
+    """q and k of a layer through one launch: bit-identical to rotating each on its own, forward and backward form, with
+    strided inputs (slices of a packed qkv projection) and position ids."""
+    s, b, nq, nk, d = 37, 2, 4, 2, 128
+    qkv = rnd(s, b, (nq + 2 * nk) * d, seed=31).to(gpu_device)
+    q = qkv[..., :nq * d].unflatten(-1, (nq, d))
+    k = qkv[..., nq * d:(nq + nk) * d].unflatten(-1, (nk, d))
+    inv = O.rope_inv_freq(d).to(gpu_device)
+    cos, sin = K.rope_table(inv, 64)
+    pos = torch.randint(0, 64, (b, s), generator=torch.Generator().manual_seed(2)).to(gpu_device)
+    for p_ids in (None, pos):
+        for backward in (False, True):
+            qo, ko = K.rope_apply_pair(q, k, cos, sin, p_ids, backward=backward)
+            assert torch.equal(qo, K.rope_apply(q, cos, sin, p_ids, backward=backward))
+            assert torch.equal(ko, K.rope_apply(k, cos, sin, p_ids, backward=backward))
+
+
 # ------------------------------------------------------------------------------------- embedding
 def test_embedding_gather_exact_and_flag(K, gpu_device):
     V, h = 1000, 256

@@ -209,6 +209,26 @@ def test_bad_token_id_raises_value_error(gpu_device):
         functional.set_input_check("sync")
 
 
+def test_position_id_beyond_the_rotary_table_raises_index_error(gpu_device):
+    """The reference indexes its cos / sin tables (one row per sequence position) with the position ids; an id past the
+    table is an indexing error there (positional_embeddings.py:109-117).  Same here, from the embedding stage."""
+    from easyllm_amd import workloads as W
+    w = dict(num_layers=1, hidden_size=256, num_attention_heads=2, num_kv_attention_heads=2, intermediate_size=512,
+             vocab_size=1024, seq=64, batch=1, seed=8)
+    model, _ = build_pair(w, gpu_device)
+    inputs, (labels, loss_mask), _ = W.make_inputs(w)
+    cu = torch.tensor([0, 40, 64])
+    good = torch.tensor([list(range(40)) + list(range(24))])
+    model(to_dev((inputs[0], good, None, cu), gpu_device))
+    bad = good.clone()
+    bad[0, 50] = 64
+    with pytest.raises(IndexError):
+        model(to_dev((inputs[0], bad, None, cu), gpu_device))
+    bad[0, 50] = -1
+    with pytest.raises(IndexError):
+        model(to_dev((inputs[0], bad, None, cu), gpu_device))
+
+
 def test_qkv_pack_and_bias_variants(gpu_device):
     """wqkv (q|k|v packed, transformer.py:427-429) with qkv bias: parity of one layer against the oracle."""
     from easyllm_amd.transformer import ParallelTransformerLayer
