@@ -22,6 +22,8 @@
 // registers one tile ahead.  dQ uses its own pass instead of atomics, so results are deterministic.
 #include "common.h"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int kThreads = 256;
@@ -288,10 +290,24 @@ __device__ __forceinline__ void load_row_frags(const bf16_t* __restrict__ rowp, 
 // =================================================================================================
 // forward
 // =================================================================================================
+// f(integral_constant<int, I>) for I = I0 .. N-1, so that the body sees its index as a constant expression
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// The loop over the key tiles below the diagonal is software-pipelined inside each wave: iteration t issues the MFMAs of
+// S(t+1) = K(t+1) Q^T and then of O += V(t) P(t), one per step, and between them the vector ALU work that turns S(t) into
+// P(t) and, once S(t+1) is complete, takes its row maxima.  A sched_barrier after every step keeps that interleaving.  The
+// K tiles therefore run one tile ahead of the V tiles in LDS.  The two tiles on the diagonal are done afterwards, one at a
+// time with the mask.
 template <int D>
 __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
     using TL = Tile<D>;
-    __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS];  // K0 V0 K1 V1
+    __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS];  // K0 V0 K1 V1: tile t of K or V in stage t & 1
     int doc_start, doc_len, qb;
     int bx, by;
     xcd_head_blocks(p.nq, bx, by);
@@ -299,7 +315,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hq = by, hk = hq / (p.nq / p.nk);
     const int q0 = qb * 128, qw0 = q0 + wave * 32;
-    const int tok_end = doc_start + doc_len;
     const int qi = qw0 + (lane & 31);                        // this lane's query (document relative)
     const int qtok = doc_start + (qi < doc_len ? qi : doc_len - 1);
     bf16x8 qf[D / 16];
@@ -307,28 +322,30 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
 
     const int kend = (q0 + 128 < doc_len ? q0 + 128 : doc_len);
     const int ntiles = (kend + 63) / 64;
+    const int nmain = 2 * qb;  // tiles wholly below the diagonal for every query of the workgroup
     const int64_t kh = (int64_t)hk * D;
     const bf16_t* kbase = p.k + tok_off(doc_start, p.s_len, p.k_ss, p.k_sb) + kh;
     const bf16_t* vbase = p.v + tok_off(doc_start, p.s_len, p.v_ss, p.v_sb) + kh;
-    // K / V tiles go from global memory straight into LDS, one tile ahead of the one being worked on
     typename TL::template Direct<kThreads / 64> kld, vld;
     kld.init(p.k_ss, lane, wave, 63);
     vld.init(p.v_ss, lane, wave, 63);
-    auto issue_tile = [&](int t, int stage) {
+    // which: 0 = K tile t, 1 = V tile t
+    auto issue_one = [&](int t, int which) {
         const int row0 = t * 64;
-        bf16_t* sk = smem + stage * 2 * TL::ELEMS;
+        bf16_t* dst = smem + (t & 1) * 2 * TL::ELEMS + which * TL::ELEMS;
+        const bf16_t* src = (which ? vbase + (int64_t)row0 * p.v_ss : kbase + (int64_t)row0 * p.k_ss);
         if (row0 + 64 <= doc_len) {
-            kld.issue(kbase + (int64_t)row0 * p.k_ss, sk, wave);
-            vld.issue(vbase + (int64_t)row0 * p.v_ss, sk + TL::ELEMS, wave);
+            if (which) vld.issue(src, dst, wave);
+            else kld.issue(src, dst, wave);
         } else {  // the document's ragged last tile: rows past its end re-read its last row
-            typename TL::template Direct<kThreads / 64> ke, ve;
-            ke.init(p.k_ss, lane, wave, doc_len - 1 - row0);
-            ve.init(p.v_ss, lane, wave, doc_len - 1 - row0);
-            ke.issue(kbase + (int64_t)row0 * p.k_ss, sk, wave);
-            ve.issue(vbase + (int64_t)row0 * p.v_ss, sk + TL::ELEMS, wave);
+            typename TL::template Direct<kThreads / 64> e;
+            e.init(which ? p.v_ss : p.k_ss, lane, wave, doc_len - 1 - row0);
+            e.issue(src, dst, wave);
         }
     };
-    issue_tile(0, 0);
+    issue_one(0, 0);
+    issue_one(0, 1);
+    if (ntiles > 1) issue_one(1, 0);
     // every load issued so far (the per-lane operand rows included) has landed before the loop starts
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
@@ -342,42 +359,132 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
     const float sl2 = p.scale * kLog2e;
     const float tau = 8.0f / sl2;  // 2^8 in units of the raw scores
 
-    for (int t = 0; t < ntiles; ++t) {
-        const int cur = t & 1;
-        const bf16_t* sK = smem + cur * 2 * TL::ELEMS;
-        const bf16_t* sV = sK + TL::ELEMS;
-        if (t + 1 < ntiles) issue_tile(t + 1, cur ^ 1);  // that stage was last read before the barrier that ended tile t-1
-        const int key0 = t * 64;
-        if (key0 <= qw0 + 31) {  // otherwise every key of the tile is after every query of this wave
-            // S^T = K Q^T in groups of 4 MFMAs; the K fragments of the next group are in flight meanwhile
-            constexpr int KG = D / 64, NG = 2 * KG;
-            f32x16 sacc[2];
-            bf16x8 fk[2][4];
-            auto ldk = [&](int g, int buf) {
+    constexpr int KD = D / 16;   // K fragments per 32 keys
+    constexpr int NKF = 2 * KD;  // K fragments of a tile
+    constexpr int NVF = 4 * (D / 32);  // V fragments of a tile
+    constexpr int NSTEP = NKF + NVF;
+    auto scores1 = [&](int t, f32x16 (&s)[2]) {
+        const bf16_t* sK = smem + (t & 1) * 2 * TL::ELEMS;
+        bf16x8 fk[2][4];
+        constexpr int KG = D / 64, NG = 2 * KG;
+        auto ldk = [&](int g, int buf) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) fk[buf][i] = TL::frag_kc(sK, (g / KG) * 32, (g % KG) * 4 + i, lane);
+            for (int i = 0; i < 4; ++i) fk[buf][i] = TL::frag_kc(sK, (g / KG) * 32, (g % KG) * 4 + i, lane);
+        };
+        ldk(0, 0);
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[kb][r] = 0.f;
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            if (g + 1 < NG) ldk(g + 1, (g + 1) & 1);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                s[g / KG] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk[g & 1][i], qf[(g % KG) * 4 + i], s[g / KG], 0, 0, 0);
+        }
+    };
+    auto rowmax = [&](const f32x16 (&s)[2]) {
+        float v = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) v = fmaxf(v, s[kb][r]);
+        return fmaxf(v, __shfl_xor(v, 32, 64));
+    };
+    // The reference point m of the exponentials only has to bound them, not equal the running maximum: it is moved (and
+    // O, l rescaled) only when some row of the wave has outgrown it by more than a factor 2^8, which after the first tiles
+    // is rare.  Probabilities then reach at most 2^8 before the final division by l.
+    auto rescale = [&](float mloc) {
+        const float mnew = fmaxf(m, mloc);
+        const float alpha = __builtin_amdgcn_exp2f((m - (mnew == -INFINITY ? 0.f : mnew)) * sl2);  // m = -inf: 0
+        lsum *= alpha;
+#pragma unroll
+        for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+        m = mnew;
+    };
+
+    f32x16 cur[2], nxt[2];
+    scores1(0, cur);  // tile 0 concerns every wave
+    float mloc = rowmax(cur);
+    bool need = true;
+    for (int t = 0; t < nmain; ++t) {
+        if (need) rescale(mloc);
+        if (t + 2 < ntiles) issue_one(t + 2, 0);  // K stage t & 1: K(t) was last read before the previous barrier
+        issue_one(t + 1, 1);                      // V stage (t+1) & 1: V(t-1) likewise; t + 1 <= nmain < ntiles
+        {
+            const bf16_t* sK = smem + ((t + 1) & 1) * 2 * TL::ELEMS;
+            const bf16_t* sV = smem + (t & 1) * 2 * TL::ELEMS + TL::ELEMS;
+            const float moff = m * sl2;
+            float ps = 0.f, mx = -INFINITY;
+            bf16x8 pf[4];
+            bf16x8 fr[4];
+            auto frag = [&](int i) {
+                if (i < NKF) return TL::frag_kc(sK, (i / KD) * 32, i % KD, lane);
+                const int j = i - NKF;
+                return TL::frag_tr(sV, (j / (D / 32)) * 16, (j % (D / 32)) * 32, lane);
             };
-            ldk(0, 0);
+            fr[0] = frag(0);
+            fr[1] = frag(1);
+            fr[2] = frag(2);
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+                for (int r = 0; r < 16; ++r) nxt[kb][r] = 0.f;
+            static_for<0, NSTEP>([&](auto ST) {
+                constexpr int i = decltype(ST)::value;
+                if constexpr (i + 3 < NSTEP) fr[(i + 3) % 4] = frag(i + 3);
+                if constexpr (i < NKF) {
+                    nxt[i / KD] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[i % 4], qf[i % KD], nxt[i / KD], 0, 0, 0);
+                } else {
+                    constexpr int j = i - NKF;
+                    oacc[j % (D / 32)] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[i % 4], pf[j / (D / 32)], oacc[j % (D / 32)], 0, 0, 0);
+                }
+                // P(t): the 32 probabilities of this lane, 32 / NKF per step during the first NKF steps (16 keys' worth,
+                // one B operand of the O MFMAs, every NKF / 4 steps)
+                if constexpr (i < NKF) {
+                    constexpr int per = 32 / NKF;  // probabilities per step
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                if (g + 1 < NG) ldk(g + 1, (g + 1) & 1);
+                    for (int n = i * per; n < (i + 1) * per; ++n)
+                        cur[n / 16][n % 16] = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[n / 16][n % 16], sl2, -moff));
+                }
+                // the sums and the conversion to bf16 trail the exponentials by one step, so that no instruction waits for
+                // the result of the one before it
+                if constexpr (i >= 1 && i <= NKF) {
+                    constexpr int per = 32 / NKF;
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    sacc[g / KG] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk[g & 1][i], qf[(g % KG) * 4 + i], sacc[g / KG], 0, 0, 0);
-            }
-            // keep that order: the reads of group g+1 are issued before the MFMAs of group g
-            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                    for (int n = (i - 1) * per; n < i * per; ++n) {
+                        const int g = n / 8, e = n % 8;
+                        ps += cur[n / 16][n % 16];
+                        pf[g][e] = (bf16_t)cur[n / 16][n % 16];
+                    }
+                }
+                if constexpr (i >= NKF) {  // S(t+1) is complete: out of the accumulators, and its maximum
+                    constexpr int per = 32 / NVF;
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                if (g + 1 < NG) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            // first V^T fragments: their LDS latency hides under the softmax arithmetic
+                    for (int n = (i - NKF) * per; n < (i - NKF + 1) * per; ++n) {
+                        cur[n / 16][n % 16] = nxt[n / 16][n % 16];
+                        mx = fmaxf(mx, cur[n / 16][n % 16]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            lsum += ps;
+            mloc = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            need = __builtin_amdgcn_ballot_w64(mloc > m + tau) != 0;
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of the tiles in flight are in LDS
+        __syncthreads();
+    }
+    // ---- the tiles on the diagonal; cur holds S(nmain) ----
+    for (int t = nmain; t < ntiles; ++t) {
+        if (t + 2 < ntiles) issue_one(t + 2, 0);
+        if (t + 1 < ntiles) issue_one(t + 1, 1);
+        const bf16_t* sV = smem + (t & 1) * 2 * TL::ELEMS + TL::ELEMS;
+        const int key0 = t * 64;
+        if (key0 <= qw0 + 31) {  // otherwise every key of the tile is after every query of this wave
             bf16x8 fv[2][D / 32];
             auto ldv = [&](int g, int buf) {
 #pragma unroll
@@ -389,35 +496,18 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
-                        if (key0 + kb * 32 + acc_row(r, lane) > qi) sacc[kb][r] = -INFINITY;
+                        if (key0 + kb * 32 + acc_row(r, lane) > qi) cur[kb][r] = -INFINITY;
             }
-            float mloc = -INFINITY;  // running maximum is kept on the raw (unscaled) scores
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) mloc = fmaxf(mloc, sacc[kb][r]);
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
-            // The reference point m of the exponentials only has to bound them, not equal the running maximum: it is moved
-            // (and O, l rescaled) only when some row of the wave has outgrown it by more than a factor 2^8, which after
-            // the first tiles is rare.  Probabilities then reach at most 2^8 before the final division by l.
-            if (__builtin_amdgcn_ballot_w64(mloc > m + tau) != 0) {
-                const float mnew = fmaxf(m, mloc);
-                const float alpha = __builtin_amdgcn_exp2f((m - (mnew == -INFINITY ? 0.f : mnew)) * sl2);  // m = -inf: 0
-                lsum *= alpha;
-#pragma unroll
-                for (int i = 0; i < D / 32; ++i)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
-                m = mnew;
-            }
+            const float ml = rowmax(cur);
+            if (__builtin_amdgcn_ballot_w64(ml > m + tau) != 0) rescale(ml);
             const float moff = (m == -INFINITY ? 0.f : m) * sl2;
             float psum = 0.f;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][r], sl2, -moff));
-                    sacc[kb][r] = pe;
+                    const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[kb][r], sl2, -moff));
+                    cur[kb][r] = pe;
                     psum += pe;
                 }
             lsum += psum;
@@ -425,13 +515,14 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 if (g + 1 < 4) ldv(g + 1, (g + 1) & 1);
-                const bf16x8 pf = acc_to_b(sacc[g >> 1], g & 1);
+                const bf16x8 pfr = acc_to_b(cur[g >> 1], g & 1);
 #pragma unroll
                 for (int db = 0; db < D / 32; ++db)
-                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv[g & 1][db], pf, oacc[db], 0, 0, 0);
+                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fv[g & 1][db], pfr, oacc[db], 0, 0, 0);
             }
         }
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of the next tile are in LDS
+        if (t + 1 < ntiles && (t + 1) * 64 <= qw0 + 31) scores1(t + 1, cur);  // K(t+1) arrived before the previous barrier
+        __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
     }
     const float ltot = lsum + __shfl_xor(lsum, 32, 64);

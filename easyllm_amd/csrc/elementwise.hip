@@ -191,25 +191,43 @@ __global__ __launch_bounds__(kBlock) void embed_count_kernel(const int64_t* __re
     }
 }
 
-// off = exclusive prefix sum of cnt over V entries: one block, each thread a contiguous run
+// off = exclusive prefix sum of cnt over V entries.  One block walks the table in chunks of 4 entries per thread (consecutive
+// threads on consecutive entries, so the accesses coalesce): a scan inside each wave, the wave totals through LDS, and the
+// running total carried from chunk to chunk.
 __global__ __launch_bounds__(kScanThreads) void embed_scan_kernel(const int* __restrict__ cnt, int* __restrict__ off, int64_t V) {
-    __shared__ int part[kScanThreads];
-    const int64_t per = (V + kScanThreads - 1) / kScanThreads;
-    const int64_t lo = (int64_t)threadIdx.x * per, hi = lo + per < V ? lo + per : V;
-    int sum = 0;
-    for (int64_t i = lo; i < hi; ++i) sum += cnt[i];
-    part[threadIdx.x] = sum;
-    __syncthreads();
-    for (int d = 1; d < kScanThreads; d <<= 1) {  // inclusive scan of the per-thread sums
-        const int v = threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+    __shared__ int wsum[kScanThreads / 64];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    int carry = 0;
+    for (int64_t base = 0; base < V; base += 4 * kScanThreads) {
+        const int64_t i0 = base + 4 * tid;
+        int c[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c[j] = i0 + j < V ? cnt[i0 + j] : 0;
+        const int mine = c[0] + c[1] + c[2] + c[3];
+        int incl = mine;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += v;
+        }
+        __syncthreads();  // the wave totals of the previous chunk have been read
+        if (lane == 63) wsum[wv] = incl;
         __syncthreads();
-        part[threadIdx.x] += v;
-        __syncthreads();
-    }
-    int run = part[threadIdx.x] - sum;
-    for (int64_t i = lo; i < hi; ++i) {
-        off[i] = run;
-        run += cnt[i];
+        int before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < kScanThreads / 64; ++w) {
+            const int v = wsum[w];
+            before += w < wv ? v : 0;
+            total += v;
+        }
+        int run = carry + before + incl - mine;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (i0 + j < V) {
+                off[i0 + j] = run;
+                run += c[j];
+            }
+        carry += total;
     }
 }
 
