@@ -144,7 +144,7 @@ def test_embedding_gather_exact_and_flag(K, gpu_device):
         O.embedding(bad, W)
 
 
-@pytest.mark.parametrize("V,h,shape", [(50, 64, (3, 200)), (7, 4096, (1, 700)), (300, 8200, (2, 150))])
+@pytest.mark.parametrize("V,h,shape", [(50, 64, (3, 200)), (7, 4096, (1, 700)), (300, 8200, (2, 150)), (9001, 64, (2, 3000))])
 def test_embedding_scatter_add(K, gpu_device, V, h, shape):
     """Heavy id collisions (V << rows); the sum per id runs in row order in fp32, so the result is bit-exact
     against a sequential fp32 loop, adds onto what the buffer already holds, and repeats identically."""
