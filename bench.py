@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the llama decoder-layer training step (fwd + loss + bwd) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--no-cpu-baseline] [--other-workloads C1,C3,C4,C5]
 
 Prints ONE JSON line.  A step = one forward + cross-entropy loss + backward of the workload's layer
 stack on one micro-batch of synthetic, HBM-resident inputs (random-init weights, seeded token ids);
@@ -13,6 +13,8 @@ launch durations, taken with events on the launch stream in a second pass of the
 events serialise the queue, so the pass that `value` is computed from runs without them).
 `cpu_baseline` = the fp32 CPU oracle (a port of the reference math) timed on this host's cores: one whole fwd+bwd step of
 the workload where that is a few tens of seconds (C1, C2), else one decoder layer + LM head + loss extrapolated linearly.
+`configs` lists the other workloads, measured after the headline figures are taken, each with ms/step, tokens/s, TFLOP/s and
+the GEMM kernel's fraction of the MFMA peak.
 """
 import argparse
 import json
@@ -74,6 +76,125 @@ def cpu_baseline(w, flops):
                       "full shape; step time extrapolated as L*t_layer + t_head; %s" % (L, t_layer, t_head, note)}
 
 
+class GemmTimer:
+    """Per-launch timing of the GEMM kernel: while installed, every launch that goes through kernels.gemm or
+    kernels.linear_dgrad_multi is bracketed by two events on the launch stream and (flops, start, end) is recorded."""
+
+    def __init__(self, kernels):
+        import torch
+        self.kernels, self.torch, self.records = kernels, torch, []
+        self._gemm, self._multi = kernels.gemm, kernels.linear_dgrad_multi
+
+    def __enter__(self):
+        torch = self.torch
+
+        def gemm(A, B, M, N, K, *a, **kw):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            out = self._gemm(A, B, M, N, K, *a, **kw)
+            end.record()
+            self.records.append((2.0 * M * N * K, start, end))
+            return out
+
+        def multi(dy2ds, ws, *a, **kw):
+            same = len({dy.stride(0) for dy in dy2ds}) == 1 and len({w.stride(0) for w in ws}) == 1 and len(ws) <= 3
+            if not same:  # goes out as one kernels.gemm call per pair, each timed above
+                return self._multi(dy2ds, ws, *a, **kw)
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            out = self._multi(dy2ds, ws, *a, **kw)
+            end.record()
+            self.records.append((2.0 * dy2ds[0].shape[0] * ws[0].shape[1] * sum(w.shape[0] for w in ws), start, end))
+            return out
+
+        self.kernels.gemm, self.kernels.linear_dgrad_multi = gemm, multi
+        return self
+
+    def __exit__(self, *exc):
+        self.kernels.gemm, self.kernels.linear_dgrad_multi = self._gemm, self._multi
+        return False
+
+
+def measure(name, steps, warmup, mode, input_check):
+    """Times `steps` fwd + loss + bwd steps of workload `name` (after `warmup` untimed ones) and, in a second pass, its GEMM
+    launches.  Returns (figures, model): figures is a flat dict, the model is handed back for the optimizer timing."""
+    import torch
+    from easyllm_amd import functional, kernels, runner, workloads as W
+    dev = torch.device("cuda:0")
+    w = W.WORKLOADS[name]
+    torch.manual_seed(w["seed"])
+    model = runner.build_model({"type": "llama_custom", "kwargs": W.model_kwargs(w)})
+    runner.attach_main_grads(model)
+    functional.set_input_check(input_check)
+    inputs, labels, doc_lens = W.make_inputs(w, device=dev)
+    tokens_per_step = w["batch"] * w["seq"]
+    flops = W.step_flops(w, doc_lens)
+
+    def step():
+        runner.zero_main_grads(model)
+        return runner.forward_step(model, inputs, labels)
+
+    def timed(fn, flush):
+        """Exactly `steps` calls of fn between two device synchronisations: (last loss, wall seconds, per-step ms from
+        one event per step boundary on the compute stream)."""
+        events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        events[0].record()
+        for i in range(steps):
+            last = fn()
+            events[i + 1].record()
+        flush()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        return last, wall, [events[i].elapsed_time(events[i + 1]) for i in range(steps)]
+
+    for _ in range(warmup):
+        loss = step()
+    loss, elapsed_eager, per_step = timed(step, functional.flush_input_checks)
+    loss_value = float(loss.item())
+    elapsed = elapsed_eager
+    launch_mode = mode
+    if mode == "graph":
+        # the same kernels, captured once and replayed: no per-kernel host work, no launch gaps
+        try:
+            graphed = runner.GraphedStep(model, inputs, labels)
+        except Exception as exc:  # capture refused by the runtime: report the eager figures and say so
+            graphed = None
+            launch_mode = "eager (graph capture failed: %s)" % (str(exc).splitlines()[0][:120] if str(exc) else type(exc).__name__)
+            print("bench.py: %s" % launch_mode, file=sys.stderr)
+        if graphed is not None:
+            for _ in range(warmup):
+                graphed()
+            loss, elapsed, per_step = timed(graphed, graphed.flush)
+            assert float(loss.item()) == loss_value, "graph replay and eager step disagree"
+            del graphed
+    per_step.sort()
+    median_ms = per_step[len(per_step) // 2] if len(per_step) % 2 else 0.5 * (per_step[len(per_step) // 2 - 1] + per_step[len(per_step) // 2])
+
+    # Second pass of the same K steps with every GEMM launch bracketed by two timing events on the launch stream.  The
+    # events serialise the queue (about 20 us per launch), so they are kept out of the pass that `value` comes from.
+    with GemmTimer(kernels) as timer:
+        t1 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        functional.flush_input_checks()
+        torch.cuda.synchronize()
+        elapsed_instrumented = time.perf_counter() - t1
+    timing = timer.records
+    gemm_flops = sum(f for f, _, _ in timing)
+    gemm_ms = sum(s.elapsed_time(e) for _, s, e in timing)
+    ms_per_step = elapsed / steps * 1e3
+    fig = dict(workload=w, name=name, tokens_per_step=tokens_per_step, flops=flops, loss=loss_value, launch=launch_mode,
+               ms_per_step=ms_per_step, ms_per_step_median=median_ms, eager_ms_per_step=elapsed_eager / steps * 1e3,
+               tok_s=tokens_per_step * steps / elapsed, tflops=flops * steps / elapsed / 1e12,
+               recomputed_layers=model.recompute_count, gemm_launches=len(timing) // max(steps, 1),
+               gemm_tflops=gemm_flops / (gemm_ms * 1e-3) / 1e12 if gemm_ms > 0 else 0.0,
+               gemm_avg_launch_us=gemm_ms * 1e3 / max(len(timing), 1), gemm_share=gemm_ms / steps / ms_per_step,
+               instrumented_ms_per_step=elapsed_instrumented / steps * 1e3)
+    return fig, model
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -86,6 +207,10 @@ def main():
     ap.add_argument("--no-optimizer-step", action="store_true", help="skip the separately timed AdamW + clipping step")
     ap.add_argument("--input-check", choices=("sync", "deferred"), default="deferred",
                     help="token-id range check of the embedding: blocking like the reference, or examined one call late")
+    ap.add_argument("--other-workloads", default="C1,C3,C4,C5",
+                    help="comma-separated workloads measured after the headline one (fewer steps each) and reported in the "
+                         "`configs` array of the same JSON line; empty string to skip")
+    ap.add_argument("--other-steps", type=int, default=6)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share only (TP=1, one MI355X); --gpus %d is not supported. "
@@ -93,97 +218,31 @@ def main():
         sys.exit(2)
 
     import torch
-    from easyllm_amd import functional, kernels, runner, workloads as W
+    from easyllm_amd import workloads as W
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    w = W.WORKLOADS[args.workload]
-    torch.manual_seed(w["seed"])
-    model = runner.build_model({"type": "llama_custom", "kwargs": W.model_kwargs(w)})
-    runner.attach_main_grads(model)
-    functional.set_input_check(args.input_check)
-    inputs, labels, doc_lens = W.make_inputs(w, device=dev)
-    tokens_per_step = w["batch"] * w["seq"]
-    flops = W.step_flops(w, doc_lens)
-
-    def step():
-        runner.zero_main_grads(model)
-        return runner.forward_step(model, inputs, labels)
-
-    def timed(fn, flush):
-        """Exactly args.steps calls of fn between two device synchronisations: (last loss, wall seconds, per-step ms from
-        one event per step boundary on the compute stream)."""
-        events = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        events[0].record()
-        for i in range(args.steps):
-            last = fn()
-            events[i + 1].record()
-        flush()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        return last, wall, [events[i].elapsed_time(events[i + 1]) for i in range(args.steps)]
-
-    for _ in range(args.warmup):
-        loss = step()
-    loss, elapsed_eager, per_step = timed(step, functional.flush_input_checks)
-    loss_value = float(loss.item())
-    elapsed = elapsed_eager
-    launch_mode = args.mode
-    if args.mode == "graph":
-        # the same kernels, captured once and replayed: no per-kernel host work, no launch gaps
-        try:
-            graphed = runner.GraphedStep(model, inputs, labels)
-        except Exception as exc:  # capture refused by the runtime: report the eager figures and say so
-            graphed = None
-            launch_mode = "eager (graph capture failed: %s)" % (str(exc).splitlines()[0][:120] if str(exc) else type(exc).__name__)
-            print("bench.py: %s" % launch_mode, file=sys.stderr)
-        if graphed is not None:
-            for _ in range(args.warmup):
-                graphed()
-            loss, elapsed, per_step = timed(graphed, graphed.flush)
-            assert float(loss.item()) == loss_value, "graph replay and eager step disagree"
-            del graphed
-    per_step.sort()
-    median_ms = per_step[len(per_step) // 2] if len(per_step) % 2 else 0.5 * (per_step[len(per_step) // 2 - 1] + per_step[len(per_step) // 2])
-
-    # Second pass of the same K steps with every GEMM launch bracketed by two timing events on the launch stream.  The
-    # events serialise the queue (about 20 us per launch), so they are kept out of the pass that `value` comes from.
-    kernels.GEMM_TIMING = []
-    t1 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    functional.flush_input_checks()
-    torch.cuda.synchronize()
-    elapsed_instrumented = time.perf_counter() - t1
-    timing, kernels.GEMM_TIMING = kernels.GEMM_TIMING, None
-
-    ms_per_step = elapsed / args.steps * 1e3
-    tok_s = tokens_per_step * args.steps / elapsed
-    tflops = flops * args.steps / elapsed / 1e12
-    gemm_flops = sum(f for f, _, _ in timing)
-    gemm_ms = sum(s.elapsed_time(e) for _, s, e in timing)
-    gemm_tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12 if gemm_ms > 0 else 0.0
+    torch.cuda.set_device(torch.device("cuda:0"))
+    fig, model = measure(args.workload, args.steps, args.warmup, args.mode, args.input_check)
+    w = fig["workload"]
     out = {
-        "metric": METRIC, "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "ms_per_step_median": round(median_ms, 3),
+        "metric": METRIC, "value": round(fig["tok_s"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(fig["ms_per_step"], 3), "ms_per_step_median": round(fig["ms_per_step_median"], 3),
         "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "%s: %s" % (args.workload, w["desc"]), "tokens_per_step": tokens_per_step,
-                   "fp32_main_grads": True, "recomputed_layers": model.recompute_count,
-                   "input_id_check": args.input_check, "launch": launch_mode,
-                   "eager_ms_per_step": round(elapsed_eager / args.steps * 1e3, 3)},
-        "tflops": round(tflops, 1), "mfma_frac_end_to_end": round(tflops / PEAK_BF16_TFLOPS, 4), "loss": round(loss_value, 5),
-        "roofline": {"kernel": "gemm_kernel (bf16 MFMA GEMM, %d launches/step)" % (len(timing) // max(args.steps, 1)),
-                     "bound": "mfma", "achieved": round(gemm_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(gemm_tflops / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_HBM_BYTES_PER_LAUNCH.get(args.workload),
-                     "avg_launch_us": round(gemm_ms * 1e3 / max(len(timing), 1), 2),
-                     "share_of_step_time": round(gemm_ms / args.steps / ms_per_step, 4),
+        "config": {"workload": "%s: %s" % (args.workload, w["desc"]), "tokens_per_step": fig["tokens_per_step"],
+                   "fp32_main_grads": True, "recomputed_layers": fig["recomputed_layers"],
+                   "input_id_check": args.input_check, "launch": fig["launch"],
+                   "eager_ms_per_step": round(fig["eager_ms_per_step"], 3)},
+        "tflops": round(fig["tflops"], 1), "mfma_frac_end_to_end": round(fig["tflops"] / PEAK_BF16_TFLOPS, 4),
+        "loss": round(fig["loss"], 5),
+        "roofline": {"kernel": "gemm_kernel (bf16 MFMA GEMM, %d launches/step)" % fig["gemm_launches"],
+                     "bound": "mfma", "achieved": round(fig["gemm_tflops"], 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(fig["gemm_tflops"] / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_HBM_BYTES_PER_LAUNCH.get(args.workload),
+                     "avg_launch_us": round(fig["gemm_avg_launch_us"], 2),
+                     "share_of_step_time": round(fig["gemm_share"], 4),
                      "measured_in": "second pass of the same %d steps with two timing events per GEMM launch (%.3f ms/step)"
-                                    % (args.steps, elapsed_instrumented / args.steps * 1e3)},
+                                    % (args.steps, fig["instrumented_ms_per_step"])},
     }
     if not args.no_optimizer_step:
         # AdamW + global-norm clipping over the same parameters, timed on its own (not part of `value`): per parameter
@@ -203,8 +262,28 @@ def main():
         out["optimizer_step"] = {"ms": round(opt_ms, 3), "params": nparams, "bound": "hbm",
                                  "achieved": round(34.0 * nparams / (opt_ms * 1e-3) / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
                                  "frac": round(34.0 * nparams / (opt_ms * 1e-3) / 1e9 / 8000.0, 4)}
+        del opt
+    del model
+    # The other workloads, each with the same procedure and fewer steps: throughput, TFLOP/s of algorithmic work (recompute
+    # not counted) and the GEMM kernel's fraction of the MFMA peak.  The headline figures above are complete before these run.
+    others = [n for n in args.other_workloads.split(",") if n and n != args.workload]
+    if others:
+        out["configs"] = []
+    for n in others:
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        f, m = measure(n, args.other_steps, 2, args.mode, args.input_check)
+        del m
+        out["configs"].append({"workload": "%s: %s" % (n, f["workload"]["desc"]), "tokens_per_step": f["tokens_per_step"],
+                               "steps": args.other_steps, "warmup": 2, "launch": f["launch"],
+                               "ms_per_step": round(f["ms_per_step"], 3), "tokens_per_s": round(f["tok_s"], 1),
+                               "tflops": round(f["tflops"], 1), "mfma_frac_end_to_end": round(f["tflops"] / PEAK_BF16_TFLOPS, 4),
+                               "recomputed_layers": f["recomputed_layers"], "gemm_tflops": round(f["gemm_tflops"], 1),
+                               "gemm_frac": round(f["gemm_tflops"] / PEAK_BF16_TFLOPS, 4),
+                               "gemm_share_of_step_time": round(f["gemm_share"], 4), "loss": round(f["loss"], 5)})
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(w, flops)
+        out["cpu_baseline"] = cpu_baseline(w, fig["flops"])
     print(json.dumps(out))
 
 

@@ -24,7 +24,7 @@ SIGNATURES = {
     "ezl_rope_apply_pair": [_vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp],
     "ezl_ids_in_range": [_vp, _i64, _i64, _vp, _vp],
     "ezl_embed_gather": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp],
-    "ezl_embed_scatter_add": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp],
+    "ezl_embed_scatter_add": [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp],
     "ezl_transpose01": [_vp, _vp, _i64, _i64, _i64, _vp],
     "ezl_add": [_vp, _vp, _vp, _i64, _vp],
     "ezl_cast_bf16_to_f32": [_vp, _vp, _i64, _vp],

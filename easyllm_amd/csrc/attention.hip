@@ -410,9 +410,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
     scores1(0, cur);  // tile 0 concerns every wave
     float mloc = rowmax(cur);
     bool need = true;
+    // every wave has finished reading K(0) before the first iteration refills its stage with K(2)
+    __syncthreads();
     for (int t = 0; t < nmain; ++t) {
         if (need) rescale(mloc);
-        if (t + 2 < ntiles) issue_one(t + 2, 0);  // K stage t & 1: K(t) was last read before the previous barrier
+        // K stage t & 1: K(t) was last read by the scores of the previous iteration (t = 0: by scores1 above), i.e. before
+        // the barrier every wave has passed since
+        if (t + 2 < ntiles) issue_one(t + 2, 0);
         issue_one(t + 1, 1);                      // V stage (t+1) & 1: V(t-1) likewise; t + 1 <= nmain < ntiles
         {
             const bf16_t* sK = smem + ((t + 1) & 1) * 2 * TL::ELEMS;

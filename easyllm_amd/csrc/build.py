@@ -10,7 +10,7 @@ LIB_DIR = os.path.join(PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libezl.so")
 SOURCES = ["api.cpp", "data_index.cpp", "norm.hip", "elementwise.hip", "cross_entropy.hip", "gemm.hip", "attention.hip", "optimizer.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-munsafe-fp-atomics",
+FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
          # packed-fp32 VALU forms are kept out of generated code on purpose
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]

@@ -170,7 +170,7 @@ __global__ __launch_bounds__(kBlock) void embed_gather_kernel(const int64_t* __r
 // The owner block of an id sorts that id's bucket by row number before summing, so the order the atomics produced never
 // reaches the result.
 constexpr int kScanThreads = 1024;
-constexpr int kBucketLds = 1024;  // buckets up to this size are sorted in LDS; longer ones by repeated selection
+constexpr int kBucketLds = 1024;  // buckets up to this size are sorted in LDS by rank; longer ones through a row bitmap
 
 __global__ __launch_bounds__(kBlock) void embed_tables_init_kernel(int* __restrict__ cnt, int* __restrict__ first,
                                                                    int* __restrict__ fill, int64_t V) {
@@ -241,16 +241,24 @@ __global__ __launch_bounds__(kBlock) void embed_bucket_kernel(const int64_t* __r
     }
 }
 
+// overwrite: dW[id] = sum instead of dW[id] += sum, and the rows of ids that do not occur are zero-filled (the whole
+// [V, h] gradient is then defined by this launch: no separate fill pass).
+constexpr int kWindowRows = 8192;  // an id with more than kBucketLds rows is ordered through a bitmap over this many row numbers
+
 template <int MAXC>
 __global__ __launch_bounds__(kBlock) void embed_scatter_bucket_kernel(const int64_t* __restrict__ ids, const bf16_t* __restrict__ dY,
                                                                       float* __restrict__ dW, const int* __restrict__ cnt,
                                                                       const int* __restrict__ first, const int* __restrict__ off,
                                                                       const int* __restrict__ bucket, int64_t rows, int h,
-                                                                      int64_t V) {
+                                                                      int64_t V, int overwrite) {
+    static_assert(kWindowRows == 32 * kBlock, "one bitmap word per thread");
+    __shared__ int list[kWindowRows];  // rows of the current id in increasing order (first kBucketLds entries double as `sorted`)
     __shared__ int raw[kBucketLds];
-    __shared__ int sorted[kBucketLds];
-    __shared__ int wmin[kBlock / 64];
+    __shared__ unsigned bits[kBlock];
+    __shared__ int wtot[kBlock / 64];
+    int* sorted = list;
     const int h8 = h >> 3;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     for (int64_t t = blockIdx.x; t < rows; t += gridDim.x) {
         const int64_t id = ids[t];
         if (id < 0 || id >= V) continue;
@@ -274,6 +282,33 @@ __global__ __launch_bounds__(kBlock) void embed_scatter_bucket_kernel(const int6
                 }
             }
         };
+        // rows lst[0 .. m-1] in that order, the loads of four rows in flight at a time
+        auto add_rows = [&](const int* lst, int m) {
+            int i = 0;
+            for (; i + 4 <= m; i += 4) {
+                bf16x8 v[4][MAXC];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int64_t jj = lst[i + u];
+#pragma unroll
+                    for (int c = 0; c < MAXC; ++c) {
+                        const int col = (c * kBlock + threadIdx.x);
+                        if (col < h8) v[u][c] = ld_bf16x8(dY + jj * h + col * 8);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+#pragma unroll
+                    for (int c = 0; c < MAXC; ++c) {
+                        const int col = (c * kBlock + threadIdx.x);
+                        if (col < h8) {
+#pragma unroll
+                            for (int k = 0; k < 8; ++k) acc[c][k] += (float)v[u][c][k];
+                        }
+                    }
+            }
+            for (; i < m; ++i) add_row(lst[i]);
+        };
         if (n == 1) {
             add_row(t);
         } else if (n <= kBucketLds) {
@@ -287,28 +322,43 @@ __global__ __launch_bounds__(kBlock) void embed_scatter_bucket_kernel(const int6
                 sorted[rank] = v;
             }
             __syncthreads();
-            for (int i = 0; i < n; ++i) add_row(sorted[i]);
+            add_rows(sorted, n);
         } else {
-            int prev = -1;
-            for (int i = 0; i < n; ++i) {  // next row = the smallest bucket entry above the previous one
-                int m = 0x7fffffff;
-                for (int j = threadIdx.x; j < n; j += kBlock) {
-                    const int v = mine[j];
-                    if (v > prev && v < m) m = v;
-                }
-#pragma unroll
-                for (int o = 32; o > 0; o >>= 1) {
-                    const int other = __shfl_xor(m, o, 64);
-                    m = other < m ? other : m;
+            // A frequent id (padding, say): its rows are put in order through a bitmap over row numbers, a window of
+            // kWindowRows rows at a time -- every thread owns one 32-row word, counts its bits, and after a scan over the
+            // block writes its rows into the ordered list.  n / kBlock bucket reads per thread and window.
+            for (int64_t w0 = 0; w0 < rows; w0 += kWindowRows) {
+                __syncthreads();  // the previous window's (or id's) LDS use is over
+                bits[threadIdx.x] = 0u;
+                __syncthreads();
+                for (int i = threadIdx.x; i < n; i += kBlock) {
+                    const int64_t r = (int64_t)mine[i] - w0;
+                    if (r >= 0 && r < kWindowRows) atomicOr(&bits[r >> 5], 1u << (r & 31));
                 }
                 __syncthreads();
-                if ((threadIdx.x & 63) == 0) wmin[threadIdx.x >> 6] = m;
-                __syncthreads();
-                m = wmin[0];
+                unsigned m = bits[threadIdx.x];
+                const int mine_n = __builtin_popcount(m);
+                int incl = mine_n;
 #pragma unroll
-                for (int wv = 1; wv < kBlock / 64; ++wv) m = wmin[wv] < m ? wmin[wv] : m;
-                add_row(m);
-                prev = m;
+                for (int o = 1; o < 64; o <<= 1) {
+                    const int v = __shfl_up(incl, o, 64);
+                    if (lane >= o) incl += v;
+                }
+                if (lane == 63) wtot[wv] = incl;
+                __syncthreads();
+                int before = 0, total = 0;
+#pragma unroll
+                for (int w = 0; w < kBlock / 64; ++w) {
+                    before += w < wv ? wtot[w] : 0;
+                    total += wtot[w];
+                }
+                int pos = before + incl - mine_n;
+                while (m) {
+                    list[pos++] = (int)w0 + 32 * (int)threadIdx.x + __builtin_ctz(m);
+                    m &= m - 1;
+                }
+                __syncthreads();
+                add_rows(list, total);
             }
         }
 #pragma unroll
@@ -316,12 +366,27 @@ __global__ __launch_bounds__(kBlock) void embed_scatter_bucket_kernel(const int6
             const int col = (c * kBlock + threadIdx.x);
             if (col < h8) {
                 float* dst = dW + id * h + col * 8;
-                f32x4 lo = *reinterpret_cast<f32x4*>(dst), hi = *reinterpret_cast<f32x4*>(dst + 4);
+                f32x4 lo, hi;
+                if (overwrite) {
 #pragma unroll
-                for (int k = 0; k < 4; ++k) { lo[k] += acc[c][k]; hi[k] += acc[c][4 + k]; }
+                    for (int k = 0; k < 4; ++k) { lo[k] = acc[c][k]; hi[k] = acc[c][4 + k]; }
+                } else {
+                    lo = *reinterpret_cast<f32x4*>(dst);
+                    hi = *reinterpret_cast<f32x4*>(dst + 4);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) { lo[k] += acc[c][k]; hi[k] += acc[c][4 + k]; }
+                }
                 *reinterpret_cast<f32x4*>(dst) = lo;
                 *reinterpret_cast<f32x4*>(dst + 4) = hi;
             }
+        }
+    }
+    if (overwrite) {  // ids that do not occur: zero rows
+        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+        for (int64_t v = blockIdx.x; v < V; v += gridDim.x) {
+            if (cnt[v] != 0) continue;
+            float* dst = dW + v * h;
+            for (int i = threadIdx.x; i < (h >> 2); i += kBlock) __builtin_nontemporal_store(z, reinterpret_cast<f32x4*>(dst) + i);
         }
     }
 }
@@ -571,12 +636,13 @@ extern "C" int64_t ezl_embed_scatter_add_workspace_bytes(int64_t rows, int64_t v
 }
 
 extern "C" int ezl_embed_scatter_add(const void* ids, const void* dy, void* dweight_f32, void* workspace, int64_t workspace_bytes,
-                                     int64_t rows, int64_t h, int64_t vocab, void* stream) {
+                                     int64_t rows, int64_t h, int64_t vocab, int accumulate, void* stream) {
     EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h < (1LL << 31) && vocab > 0, EZL_EUNSUPPORTED,
                 "ezl_embed_scatter_add: h must be a multiple of 8");
     EZL_REQUIRE((rows == 0 || (ids && dy && dweight_f32)) && ezl_aligned16(dy), EZL_EINVAL,
                 "ezl_embed_scatter_add: null or misaligned pointer");
-    if (rows == 0) return EZL_OK;
+    if (rows == 0 && accumulate) return EZL_OK;
+    EZL_REQUIRE(dweight_f32, EZL_EINVAL, "ezl_embed_scatter_add: null or misaligned pointer");
     EZL_REQUIRE(h <= 8192 * 2, EZL_EUNSUPPORTED, "ezl_embed_scatter_add: h must be <= 16384");
     EZL_REQUIRE(rows < (1LL << 31) && vocab < (1LL << 31), EZL_EUNSUPPORTED, "ezl_embed_scatter_add: more than 2^31 rows or ids");
     EZL_REQUIRE(((uintptr_t)dweight_f32 & 15) == 0, EZL_EINVAL, "ezl_embed_scatter_add: dweight must be 16-byte aligned");
@@ -595,16 +661,19 @@ extern "C" int ezl_embed_scatter_add(const void* ids, const void* dy, void* dwei
     hipLaunchKernelGGL(embed_bucket_kernel, dim3(grid_for(rows, kBlock, 1024)), dim3(kBlock), 0, st, (const int64_t*)ids, off, fill,
                        bucket, rows, vocab);
     EZL_LAUNCH_CHECK("ezl_embed_scatter_add(tables)");
-    const dim3 grid(grid_for(rows, 1));
+    // one workgroup per token row (accumulate) or per vocabulary row, whichever is more: the zero fill of the rows that
+    // received nothing is most of the traffic when the result overwrites the buffer
+    const dim3 grid(grid_for(accumulate ? rows : (rows > vocab ? rows : vocab), 1));
+    const int overwrite = accumulate ? 0 : 1;
     if (h <= 8 * kBlock * 2)
         hipLaunchKernelGGL((embed_scatter_bucket_kernel<2>), grid, dim3(kBlock), 0, st, (const int64_t*)ids, (const bf16_t*)dy,
-                           (float*)dweight_f32, cnt, first, off, bucket, rows, (int)h, vocab);
+                           (float*)dweight_f32, cnt, first, off, bucket, rows, (int)h, vocab, overwrite);
     else if (h <= 8 * kBlock * 4)
         hipLaunchKernelGGL((embed_scatter_bucket_kernel<4>), grid, dim3(kBlock), 0, st, (const int64_t*)ids, (const bf16_t*)dy,
-                           (float*)dweight_f32, cnt, first, off, bucket, rows, (int)h, vocab);
+                           (float*)dweight_f32, cnt, first, off, bucket, rows, (int)h, vocab, overwrite);
     else
         hipLaunchKernelGGL((embed_scatter_bucket_kernel<8>), grid, dim3(kBlock), 0, st, (const int64_t*)ids, (const bf16_t*)dy,
-                           (float*)dweight_f32, cnt, first, off, bucket, rows, (int)h, vocab);
+                           (float*)dweight_f32, cnt, first, off, bucket, rows, (int)h, vocab, overwrite);
     EZL_LAUNCH_CHECK("ezl_embed_scatter_add");
     return EZL_OK;
 }

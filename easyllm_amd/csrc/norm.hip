@@ -5,9 +5,9 @@
 // of llama/transformer.py:786 fused in front (sum rounded to bf16 first, as the reference's bf16
 // tensor add does).
 //
-// Layout: rows of h bf16, h % 8 == 0, h <= 8192.  A row is held in registers (read from HBM exactly once) by
-// TPR = min(256, h/8 rounded up to a wave) threads whose row sums meet through a double-buffered LDS cell (forward;
-// backward for h > 4096, one barrier per row), or by one wave (backward for h <= 4096).
+// Layout: rows of h bf16, h % 8 == 0, h <= 8192.  A row is held in registers (read from HBM exactly once): forward by
+// TPR = min(256, h/8 rounded up to a wave) threads whose row sums meet through a double-buffered LDS cell; backward by one
+// wave (h <= 4096) or by a pair of waves (wider rows).
 #include "common.h"
 
 #include <mutex>
@@ -79,120 +79,7 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16_t* __restri
     }
 }
 
-// dx = rstd * (g - xhat * mean(g * xhat)),  g = dy * w, xhat = x * rstd;  dw = sum_rows dy * xhat.
-// Each thread keeps the dw partial of its own columns over all rows the block visits; the row slots
-// of a block are then folded through LDS and one partial row per block goes to HBM.
-template <int NCHUNK, bool HAS_DRES>
-__global__ __launch_bounds__(1024) void rmsnorm_bwd_kernel(const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
-                                                           const bf16_t* __restrict__ w, const float* __restrict__ rstd,
-                                                           const bf16_t* __restrict__ dres, bf16_t* __restrict__ dx,
-                                                           float* __restrict__ dw_partial, int T, int h, int tpr) {
-    extern __shared__ float fold[];  // h floats
-    __shared__ float red[2][16][4];
-    const int rpb = 1024 / tpr;
-    const int slot = threadIdx.x / tpr;
-    const int tin = threadIdx.x % tpr;
-    const int wis = tin >> 6;
-    const int nws = tpr >> 6;
-    const int lane = threadIdx.x & 63;
-    float wv[NCHUNK][8];
-    float dwacc[NCHUNK][8];
-#pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) {
-        const int col = (c * tpr + tin) * 8;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { dwacc[c][i] = 0.f; wv[c][i] = 0.f; }
-        if (col < h) unpack8(ld_bf16x8(w + col), wv[c]);
-    }
-    int parity = 0;
-    const float inv_h = 1.0f / (float)h;
-    // The operands of the block's next rows are requested before the current rows are reduced, so HBM reads stay in
-    // flight across the barrier of the row reduction.
-    bf16x8 xr[NCHUNK], dyr[NCHUNK], drr[NCHUNK];
-    auto fetch = [&](int row0, bf16x8* xo, bf16x8* dyo, bf16x8* dro) {
-        const int row = row0 + slot;
-        const size_t base = (size_t)row * h;
-#pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) {
-            const int col = (c * tpr + tin) * 8;
-            if (row < T && col < h) {
-                xo[c] = ld_bf16x8(x + base + col);
-                dyo[c] = ld_bf16x8(dy + base + col);
-                if (HAS_DRES) dro[c] = ld_bf16x8(dres + base + col);
-            }
-        }
-    };
-    const int stride = gridDim.x * rpb;
-    int row0 = blockIdx.x * rpb;
-    if (row0 < T) fetch(row0, xr, dyr, drr);
-    for (; row0 < T; row0 += stride) {
-        const int row = row0 + slot;
-        const bool live = row < T;
-        const size_t base = (size_t)row * h;
-        const float rs = live ? rstd[row] : 0.f;
-        bf16x8 xn[NCHUNK], dyn[NCHUNK], drn[NCHUNK];
-        if (row0 + stride < T) fetch(row0 + stride, xn, dyn, drn);
-        float dot = 0.f;
-#pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) {
-            const int col = (c * tpr + tin) * 8;
-            if (live && col < h) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) dot += (float)dyr[c][i] * wv[c][i] * ((float)xr[c][i] * rs);
-            }
-        }
-        dot = wave_sum(dot);
-        if (nws > 1) {
-            if (lane == 0) red[parity][slot][wis] = dot;
-            __syncthreads();
-            dot = 0.f;
-            for (int i = 0; i < nws; ++i) dot += red[parity][slot][i];
-            parity ^= 1;
-        }
-        const float cmean = dot * inv_h;
-#pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) {
-            const int col = (c * tpr + tin) * 8;
-            if (live && col < h) {
-                float o[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const float xhat = (float)xr[c][i] * rs;
-                    const float dyv = (float)dyr[c][i];
-                    o[i] = rs * (dyv * wv[c][i] - xhat * cmean);
-                    if (HAS_DRES) o[i] += (float)drr[c][i];
-                    dwacc[c][i] += dyv * xhat;
-                }
-                st_bf16x8(dx + base + col, pack8(o));
-            }
-        }
-#pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) {
-            xr[c] = xn[c];
-            dyr[c] = dyn[c];
-            if (HAS_DRES) drr[c] = drn[c];
-        }
-    }
-    // fold the row slots of this block: slot 0 stores, the others add, one barrier per slot
-    for (int s = 0; s < rpb; ++s) {
-        if (slot == s) {
-#pragma unroll
-            for (int c = 0; c < NCHUNK; ++c) {
-                const int col = (c * tpr + tin) * 8;
-                if (col < h) {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        if (s == 0) fold[col + i] = dwacc[c][i];
-                        else fold[col + i] += dwacc[c][i];
-                    }
-                }
-            }
-        }
-        __syncthreads();
-    }
-    for (int j = threadIdx.x; j < h; j += 1024) dw_partial[(size_t)blockIdx.x * h + j] = fold[j];
-}
-
+// Backward: dx = rstd * (g - xhat * mean(g * xhat)),  g = dy * w, xhat = x * rstd;  dw = sum_rows dy * xhat.
 // ---- backward with one wave per row (h <= 4096) ----------------------------------------------------------------
 // A row is owned by ONE wave: lane l holds the 8 columns (c * 64 + l) * 8 .. + 7 of chunk c, so every chunk is one
 // coalesced 1 KiB access, the row sums need wave shuffles only and there is no barrier inside the row loop: the waves
@@ -278,6 +165,99 @@ __global__ __launch_bounds__(512) void rmsnorm_bwd_wave_kernel(const bf16_t* __r
     for (int j = threadIdx.x; j < h; j += 512) dw_partial[(size_t)blockIdx.x * h + j] = fold[j];
 }
 
+// ---- backward with two waves per row (4096 < h <= 8192) -------------------------------------------------------------
+// The same scheme with a row shared by the two waves of a pair: wave half 0 owns the first NCHUNK * 512 columns, half 1 the
+// rest, so the per-lane state (operands, weight, dw partials) is that of a row of half the width and stays in registers.
+// The two partial sums of a row meet in an LDS cell (double buffered by iteration parity: one barrier per row).  A block is
+// 4 waves = 2 rows per pass, two blocks per CU: while the waves of one block wait at their barrier the other block's loads
+// are in flight.
+template <int NCHUNK, bool HAS_DRES>
+__global__ __launch_bounds__(256, 2) void rmsnorm_bwd_pair_kernel(const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
+                                                                  const bf16_t* __restrict__ w, const float* __restrict__ rstd,
+                                                                  const bf16_t* __restrict__ dres, bf16_t* __restrict__ dx,
+                                                                  float* __restrict__ dw_partial, int T, int h) {
+    extern __shared__ float fold[];  // h floats
+    __shared__ float cell[2][2][2];  // [parity][row slot][half]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform values stay in scalar registers
+    const int slot = wave >> 1, half = wave & 1;
+    const int col0 = (half * NCHUNK * 64 + lane) * 8;  // this lane's first column; chunk c is 512 c further
+    bf16x8 wr[NCHUNK];
+    float dwacc[NCHUNK][8];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+        const int col = col0 + c * 512;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { dwacc[c][i] = 0.f; wr[c][i] = (bf16_t)0.0f; }
+        if (col < h) wr[c] = ld_bf16x8(w + col);
+    }
+    const float inv_h = 1.0f / (float)h;
+    int parity = 0;
+    // every wave of the block runs the same number of iterations (barrier inside)
+    for (int row0 = blockIdx.x * 2; row0 < T; row0 += gridDim.x * 2) {
+        const int row = row0 + slot;
+        const bool live = row < T;
+        const bf16_t* xrow = x + (size_t)row * h + col0;
+        const bf16_t* dyrow = dy + (size_t)row * h + col0;
+        const float rs = live ? rstd[row] : 0.f;
+        bf16x8 xr[NCHUNK], dyr[NCHUNK], drr[NCHUNK];
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { xr[c][i] = (bf16_t)0.0f; dyr[c][i] = (bf16_t)0.0f; }
+            if (live && col0 + c * 512 < h) {
+                xr[c] = ld_bf16x8_nt(xrow + c * 512);
+                dyr[c] = ld_bf16x8_nt(dyrow + c * 512);
+                if (HAS_DRES) drr[c] = ld_bf16x8_nt(dres + (size_t)row * h + col0 + c * 512);
+            }
+        }
+        float dot = 0.f;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dot += (float)dyr[c][i] * (float)wr[c][i] * ((float)xr[c][i] * rs);
+        dot = wave_sum(dot);
+        if (lane == 0) cell[parity][slot][half] = dot;
+        __syncthreads();
+        const float cmean = (cell[parity][slot][0] + cell[parity][slot][1]) * inv_h;  // same order in both waves
+        parity ^= 1;
+        bf16_t* dxrow = dx + (size_t)row * h + col0;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            asm volatile("" : "+v"(xr[c]), "+v"(dyr[c]));  // do not keep the fp32 copies of the dot product alive
+            if (live && col0 + c * 512 < h) {
+                float o[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float xhat = (float)xr[c][i] * rs;
+                    const float dyv = (float)dyr[c][i];
+                    o[i] = rs * (dyv * (float)wr[c][i] - xhat * cmean);
+                    if (HAS_DRES) o[i] += (float)drr[c][i];
+                    dwacc[c][i] += dyv * xhat;
+                }
+                st_bf16x8_nt(dxrow + c * 512, pack8(o));
+            }
+        }
+    }
+    for (int s = 0; s < 2; ++s) {  // row slot 0 stores, slot 1 adds: a fixed order
+        if (slot == s) {
+#pragma unroll
+            for (int c = 0; c < NCHUNK; ++c) {
+                const int col = col0 + c * 512;
+                if (col < h) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        if (s == 0) fold[col + i] = dwacc[c][i];
+                        else fold[col + i] += dwacc[c][i];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    for (int j = threadIdx.x; j < h; j += 256) dw_partial[(size_t)blockIdx.x * h + j] = fold[j];
+}
+
 int tpr_for(int h) {
     int t = (h / 8 + 63) / 64 * 64;
     return t < 64 ? 64 : (t > 256 ? 256 : t);
@@ -317,9 +297,14 @@ extern "C" int ezl_rmsnorm_fwd(const void* x, const void* residual, const void* 
     return EZL_OK;
 }
 
+namespace {
+// blocks (= fp32 partial rows of h) the backward kernels want: 8 waves per CU in both forms
+int64_t rmsnorm_bwd_blocks(int64_t h) { return h <= 4096 ? 256 : 512; }
+}  // namespace
+
 extern "C" int64_t ezl_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t h) {
     (void)rows;
-    return (int64_t)256 * h * (int64_t)sizeof(float);
+    return rmsnorm_bwd_blocks(h) * h * (int64_t)sizeof(float);
 }
 
 namespace {
@@ -336,15 +321,17 @@ int rmsnorm_bwd_check(const char* name, const void* dy, const void* x, const voi
     return EZL_OK;
 }
 
-// both entry points: `partials` holds one fp32 row of h per block (at most 256 blocks), every used row fully written
+// both entry points: `partials` holds one fp32 row of h per block (at most max_blocks blocks; the narrow-row kernel uses up
+// to 256, the wide-row one up to 512), every used row fully written
 int rmsnorm_bwd_launch(const void* dy, const void* x, const void* weight, const void* rstd, const void* dresidual, void* dx,
-                       void* dw_bf16, void* dw_f32, int accumulate, float* partials, int64_t rows, int64_t h, hipStream_t st) {
+                       void* dw_bf16, void* dw_f32, int accumulate, float* partials, int64_t max_blocks, int64_t rows, int64_t h,
+                       hipStream_t st) {
     const size_t smem = (size_t)h * sizeof(float);
     int64_t grid;
     if (h <= 4096) {  // one wave per row, 8 rows per block
         const int nchunk = ((int)h + 511) / 512;
         grid = (rows + 7) / 8;
-        if (grid > 256) grid = 256;
+        if (grid > max_blocks) grid = max_blocks;
         if (grid < 1) grid = 1;  // rows == 0 still produces a zero dw
 #define LAUNCH(NC, DR)                                                                                                    \
     hipLaunchKernelGGL((rmsnorm_bwd_wave_kernel<NC, DR>), dim3((unsigned)grid), dim3(512), smem, st, (const bf16_t*)dy,    \
@@ -360,22 +347,23 @@ int rmsnorm_bwd_launch(const void* dy, const void* x, const void* weight, const 
         if (dresidual) LAUNCH_NC(true); else LAUNCH_NC(false);
 #undef LAUNCH_NC
 #undef LAUNCH
-    } else {  // wider rows: 256 threads per row, row sums across waves through LDS
-        const int tpr = tpr_for((int)h);
-        const int nchunk = ((int)h + tpr * 8 - 1) / (tpr * 8);
-        const int rpb = 1024 / tpr;
-        grid = (rows + rpb - 1) / rpb;
-        if (grid > 256) grid = 256;
+    } else {  // wider rows: two waves per row, 2 rows per block pass, two blocks per CU
+        const int nchunk = ((int)h + 1023) / 1024;  // 512-column chunks per wave
+        grid = (rows + 1) / 2;
+        if (grid > max_blocks) grid = max_blocks;
         if (grid < 1) grid = 1;
-#define LAUNCH(NC, DR)                                                                                            \
-    hipLaunchKernelGGL((rmsnorm_bwd_kernel<NC, DR>), dim3((unsigned)grid), dim3(1024), smem, st, (const bf16_t*)dy, \
-                       (const bf16_t*)x, (const bf16_t*)weight, (const float*)rstd, (const bf16_t*)dresidual,     \
-                       (bf16_t*)dx, partials, (int)rows, (int)h, tpr)
-        if (dresidual) {
-            if (nchunk == 1) LAUNCH(1, true); else if (nchunk == 2) LAUNCH(2, true); else LAUNCH(4, true);
-        } else {
-            if (nchunk == 1) LAUNCH(1, false); else if (nchunk == 2) LAUNCH(2, false); else LAUNCH(4, false);
-        }
+#define LAUNCH(NC, DR)                                                                                                    \
+    hipLaunchKernelGGL((rmsnorm_bwd_pair_kernel<NC, DR>), dim3((unsigned)grid), dim3(256), smem, st, (const bf16_t*)dy,    \
+                       (const bf16_t*)x, (const bf16_t*)weight, (const float*)rstd, (const bf16_t*)dresidual, (bf16_t*)dx, \
+                       partials, (int)rows, (int)h)
+#define LAUNCH_NC(DR)                                  \
+    do {                                               \
+        if (nchunk <= 5) LAUNCH(5, DR);                \
+        else if (nchunk <= 6) LAUNCH(6, DR);           \
+        else LAUNCH(8, DR);                            \
+    } while (0)
+        if (dresidual) LAUNCH_NC(true); else LAUNCH_NC(false);
+#undef LAUNCH_NC
 #undef LAUNCH
     }
     EZL_LAUNCH_CHECK("ezl_rmsnorm_bwd");
@@ -393,20 +381,20 @@ extern "C" int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight
     if (const int rc = rmsnorm_bwd_check("ezl_rmsnorm_bwd", dy, x, weight, rstd, dresidual, dx, dw_bf16, dw_f32, rows, h)) return rc;
     EZL_REQUIRE(workspace && workspace_bytes >= ezl_rmsnorm_bwd_workspace_bytes(rows, h), EZL_EINVAL,
                 "ezl_rmsnorm_bwd: workspace missing or too small");
-    return rmsnorm_bwd_launch(dy, x, weight, rstd, dresidual, dx, dw_bf16, dw_f32, accumulate, (float*)workspace, rows, h,
-                              (hipStream_t)stream);
+    return rmsnorm_bwd_launch(dy, x, weight, rstd, dresidual, dx, dw_bf16, dw_f32, accumulate, (float*)workspace,
+                              rmsnorm_bwd_blocks(h), rows, h, (hipStream_t)stream);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
 // ezl_rmsnorm_bwd without a workspace argument, for callers that cannot obtain device memory (code under HIP graph
 // capture, serving loops, harnesses that forbid allocation): the per-block dw partials live in a file-scope device array
-// of the largest size the kernels can need (256 blocks x h <= 8192 floats = 8 MiB), held by every GPU the library runs on
+// of the largest size the kernels can need (512 blocks x h <= 8192 floats = 16 MiB), held by every GPU the library runs on
 // until the process ends.  All calls on one GPU share that array: calls that overlap on one GPU (different streams or
 // host threads) race on it.  Nothing in it needs clearing: every row of partials that is read has been written by the
 // same call.
 namespace {
 
-constexpr int kScratchBlocks = 256, kScratchMaxH = 8192;
+constexpr int kScratchBlocks = 512, kScratchMaxH = 8192;
 constexpr int kMaxDevices = 64;
 static __device__ __align__(256) float scratch[kScratchBlocks * kScratchMaxH];
 
@@ -415,13 +403,18 @@ static __device__ __align__(256) float scratch[kScratchBlocks * kScratchMaxH];
 float* g_scratch_ptr[kMaxDevices] = {};
 std::mutex g_scratch_mutex;
 
-int scratch_for_current_device(float** out) {
+int scratch_for_current_device(float** out, hipStream_t stream) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     EZL_REQUIRE(e == hipSuccess && dev >= 0 && dev < kMaxDevices, EZL_EHIP, "ezl_rmsnorm_bwd_noalloc: cannot identify the current device (%s)",
                 hipGetErrorString(e));
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (!g_scratch_ptr[dev]) {
+        // The lookup is a runtime call that may load the code object: not something to do while the stream records a graph.
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        e = hipStreamIsCapturing(stream, &cap);
+        EZL_REQUIRE(e == hipSuccess && cap == hipStreamCaptureStatusNone, EZL_EINVAL,
+                    "ezl_rmsnorm_bwd_noalloc: the first call on a device must not be made under stream capture (call it once before)");
         void* p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         EZL_REQUIRE(e == hipSuccess && p, EZL_EHIP, "ezl_rmsnorm_bwd_noalloc: hipGetSymbolAddress failed (%s)", hipGetErrorString(e));
@@ -440,9 +433,9 @@ extern "C" int ezl_rmsnorm_bwd_noalloc(const void* dy, const void* x, const void
     EZL_REQUIRE(h <= kScratchMaxH, EZL_EUNSUPPORTED, "ezl_rmsnorm_bwd_noalloc: h = %lld exceeds the built-in scratch (h <= %d)",
                 (long long)h, kScratchMaxH);
     if (const int rc = rmsnorm_bwd_check("ezl_rmsnorm_bwd_noalloc", dy, x, weight, rstd, dresidual, dx, dw_bf16, dw_f32, rows, h)) return rc;
-    EZL_REQUIRE(ezl_rmsnorm_bwd_workspace_bytes(rows, h) <= (int64_t)sizeof(float) * kScratchBlocks * kScratchMaxH, EZL_EUNSUPPORTED,
-                "ezl_rmsnorm_bwd_noalloc: problem exceeds the built-in scratch");
+    const int64_t blocks = rmsnorm_bwd_blocks(h);  // as in ezl_rmsnorm_bwd, so that both give the same bits
+    static_assert(kScratchBlocks >= 512, "the scratch holds the partial rows of the widest launch");
     float* partials = nullptr;
-    if (const int rc = scratch_for_current_device(&partials)) return rc;
-    return rmsnorm_bwd_launch(dy, x, weight, rstd, dresidual, dx, dw_bf16, dw_f32, accumulate, partials, rows, h, (hipStream_t)stream);
+    if (const int rc = scratch_for_current_device(&partials, (hipStream_t)stream)) return rc;
+    return rmsnorm_bwd_launch(dy, x, weight, rstd, dresidual, dx, dw_bf16, dw_f32, accumulate, partials, blocks, rows, h, (hipStream_t)stream);
 }

@@ -332,12 +332,10 @@ class EmbeddingFunction(torch.autograd.Function):
         ids, weight = ctx.saved_tensors
         mg, acc = _main_grad_target(weight)
         if mg is not None:
-            if not acc:
-                mg.zero_()
-            K.embed_scatter_add(ids, dout.contiguous(), mg)
+            K.embed_scatter_add(ids, dout.contiguous(), mg, accumulate=acc)
             return None, None
-        buf = torch.zeros(weight.shape, dtype=torch.float32, device=weight.device)
-        K.embed_scatter_add(ids, dout.contiguous(), buf)
+        buf = torch.empty(weight.shape, dtype=torch.float32, device=weight.device)
+        K.embed_scatter_add(ids, dout.contiguous(), buf, accumulate=False)
         return None, K.cast_f32_to_bf16(buf)
 
 

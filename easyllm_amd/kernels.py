@@ -177,14 +177,16 @@ def embed_gather(ids, weight):
     return out, flag
 
 
-def embed_scatter_add(ids, dy, dweight_f32):
+def embed_scatter_add(ids, dy, dweight_f32, accumulate=True):
+    """dweight_f32[id] (+)= sum of the dy rows of that id, in row order.  accumulate=False overwrites the buffer: rows of
+    ids that do not occur come back zero."""
     _need(ids.is_cuda and ids.dtype == torch.int64 and ids.is_contiguous(), "ids must be contiguous int64 on the GPU")
     _bf16c(dy, "dy")
     V, h = dweight_f32.shape
     _need(dweight_f32.dtype == torch.float32 and dweight_f32.is_contiguous() and dy.shape[-1] == h, "bad dweight")
     ws_bytes = _lib.embed_scatter_add_workspace_bytes(ids.numel(), V)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dy.device)
-    _lib.call("ezl_embed_scatter_add", _p(ids), _p(dy), _p(dweight_f32), _p(ws), ws_bytes, ids.numel(), h, V, _stream())
+    _lib.call("ezl_embed_scatter_add", _p(ids), _p(dy), _p(dweight_f32), _p(ws), ws_bytes, ids.numel(), h, V, 1 if accumulate else 0, _stream())
 
 
 # ------------------------------------------------------------------------------------- plumbing
@@ -227,20 +229,7 @@ def _rows_ld(t, name):
     return t.stride(0)
 
 
-# Optional per-launch timing of the GEMM kernel (used by bench.py for the roofline figure): when a list
-# is installed here every launch is bracketed by two events on the launch stream and
-# (flops, start, end) is appended to it.
-GEMM_TIMING = None
-
-
 def gemm(A, B, M, N, K, lda, ldb, a_kc, b_kc, out=None, out_dtype=BF16, accumulate=False):
-    if GEMM_TIMING is not None:
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        out = _gemm(A, B, M, N, K, lda, ldb, a_kc, b_kc, out, out_dtype, accumulate)
-        end.record()
-        GEMM_TIMING.append((2.0 * M * N * K, start, end))
-        return out
     return _gemm(A, B, M, N, K, lda, ldb, a_kc, b_kc, out, out_dtype, accumulate)
 
 
@@ -307,15 +296,9 @@ def linear_dgrad_multi(dy2ds, ws, out=None, accumulate=False):
     if out is None:
         out = torch.empty(T, n_in, dtype=BF16, device=dy2ds[0].device)
     _need(out.is_cuda and out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (T, n_in) and out.dtype == BF16, "bad GEMM output")
-    if GEMM_TIMING is not None:
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
     _lib.call("ezl_gemm_bf16_ksplit", n, (ctypes.c_void_p * n)(*[_p(dy) for dy in dy2ds]), (ctypes.c_void_p * n)(*[_p(w) for w in ws]),
               _p(out), T, n_in, (ctypes.c_int64 * n)(*[w.shape[0] for w in ws]), ldas[0], ldbs[0], out.stride(0), 1, 0, 0,
               1 if accumulate else 0, _stream())
-    if GEMM_TIMING is not None:
-        end.record()
-        GEMM_TIMING.append((2.0 * T * n_in * sum(w.shape[0] for w in ws), start, end))
     return out
 
 

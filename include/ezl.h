@@ -6,12 +6,16 @@
  *
  * Conventions
  *   - every pointer is a DEVICE pointer unless stated otherwise; buffers are owned by the caller;
- *     nothing here allocates or frees device memory; workspaces are passed in;
+ *     nothing here allocates or frees device memory; workspaces are passed in (one exception:
+ *     ezl_rmsnorm_bwd_noalloc keeps its workspace in a device array of the library itself);
  *   - bf16 tensors: base 16-byte aligned, innermost dimension contiguous and a multiple of 8;
  *   - `stream` is a hipStream_t (NULL = default stream); all work is enqueued there, no host sync;
  *   - return 0 on success, a negative EZL_E* code otherwise; ezl_last_error() returns the message
  *     of the last failure on the calling thread;
  *   - re-entrant: no global mutable state; callable from any host thread (autograd workers included).
+ *     The exception again is ezl_rmsnorm_bwd_noalloc, whose calls on one GPU share one array.
+ *   - the code object is gfx950 only (64-wide waves, 160 KiB of LDS per workgroup; several kernels use
+ *     more than 64 KiB): on any other GPU the first launch fails with EZL_EHIP.
  */
 #ifndef EZL_H
 #define EZL_H
@@ -43,7 +47,7 @@ int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const voi
 
 /* ezl_rmsnorm_bwd without the workspace argument.  No counterpart in the reference: it exists for callers that cannot
  * obtain device memory at the call site (code under HIP graph capture, tight serving loops, harnesses that forbid
- * allocation).  The per-block dw partials go to a device array built into the library (8 MiB per GPU, held until the
+ * allocation).  The per-block dw partials go to a device array built into the library (16 MiB per GPU, held until the
  * process ends), which covers every shape ezl_rmsnorm_bwd accepts (h <= ezl_rmsnorm_bwd_noalloc_max_h() = 8192); a larger
  * h is refused with EZL_EUNSUPPORTED.  Same kernels and bit-identical results as ezl_rmsnorm_bwd.  All calls on one GPU
  * share the array: calls that overlap on one GPU (other streams or host threads) race.  The first call on a device looks
@@ -78,14 +82,17 @@ int ezl_rope_apply_pair(const void* q, void* q_out, int64_t nq, int64_t q_in_str
 /* ---- token embedding: base_modules/layers/vocab_parallel_emb.py:106-137 (F.embedding, TP=1) ----
  * gather: out[r] = weight[ids[r]] (bit-exact row copy); an id outside [0, vocab) ORs 1 (id >= vocab)
  * or 2 (id < 0) into *bad_flag (device int32) and yields a zero row.
- * scatter_add: dweight_f32[id] += sum of dy[r] over rows with ids[r] == id, fp32, added in increasing row order whatever
- * the launch does (bit-reproducible), in time linear in `rows`; workspace: ezl_embed_scatter_add_workspace_bytes(rows, vocab)
- * bytes of device memory, 4-byte aligned, contents irrelevant before and after. */
+ * scatter_add: dweight_f32[id] (+)= sum of dy[r] over rows with ids[r] == id, fp32, added in increasing row order whatever
+ * the launch does (bit-reproducible).  accumulate != 0 adds to what the buffer holds; accumulate == 0 overwrites it and
+ * zero-fills the rows of ids that do not occur, so the whole [vocab, h] gradient is written by the call.  Work is linear
+ * in `rows`; an id that occurs n > 1024 times is summed by one workgroup in n consecutive row visits.  workspace:
+ * ezl_embed_scatter_add_workspace_bytes(rows, vocab) bytes of device memory, 4-byte aligned, contents irrelevant before
+ * and after. */
 int ezl_embed_gather(const void* ids, const void* weight, void* out, void* bad_flag, int64_t rows, int64_t h, int64_t vocab,
                      void* stream);
 int64_t ezl_embed_scatter_add_workspace_bytes(int64_t rows, int64_t vocab);
 int ezl_embed_scatter_add(const void* ids, const void* dy, void* dweight_f32, void* workspace, int64_t workspace_bytes,
-                          int64_t rows, int64_t h, int64_t vocab, void* stream);
+                          int64_t rows, int64_t h, int64_t vocab, int accumulate, void* stream);
 
 /* ---- layout / dtype plumbing of llama/llama.py:145-188 (transpose, undo, float16_to_fp32) ---- */
 int ezl_transpose01(const void* x, void* y, int64_t d0, int64_t d1, int64_t inner, void* stream); /* y[j,i,:] = x[i,j,:] */

@@ -11,13 +11,16 @@ decisions decorrelate within a few ops -- tests/test_oracle.py shows it on the C
 trajectory that a correct implementation could follow.)
 
 Rule: a tensor passes if it meets the stated bar against the fp32 oracle; where it does not, it passes only if it is no
-farther from the fp32 oracle than the bf16-storage evaluation of the same computation is (relative L2 within 15 %, largest
-error within 50 %: an extreme value over up to 10^8 elements).  Every figure is printed either way.
+farther from the fp32 oracle than the bf16-storage evaluation of the same computation is (relative L2 within 5 %, largest
+error within 25 %: an extreme value over up to 10^8 elements; the widest margins seen on the full-size workloads are 2.5 %
+and 11 %).  Every figure is printed either way.  tests/test_oracle.py checks the bf16-storage evaluation itself against an
+independent bf16 implementation (transformers' LlamaForCausalLM run in bf16) at the headline workload's widths through the
+distances committed in tests/golden/bf16_floor_c2_widths.json.
 """
 import torch
 
 REL, COS = 2e-2, 0.9999
-L2_SLACK, MAX_SLACK = 1.15, 1.5
+L2_SLACK, MAX_SLACK = 1.05, 1.25
 
 
 def gap(a, ref):

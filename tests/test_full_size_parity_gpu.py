@@ -1,4 +1,4 @@
-"""Parity of the full-size benchmark workloads (C2, C3, C4) with the CPU oracle, run on the host cores of the GPU box
+"""Parity of the full-size benchmark workloads (C2, C3, C4, and layers 0 and 7 + head of the packed C5) with the CPU oracle, run on the host cores of the GPU box
 on the same weights, token ids and labels.  The comparison rule (stated bar against the fp32 oracle; where a chain of
 bf16-stored ops cannot meet it, no farther from fp32 than the oracle's exact-arithmetic bf16-storage evaluation) is in
 tests/_parity.py.
@@ -53,9 +53,12 @@ def _hip_step(name, dev):
         def fwd(module, args, out):
             x_in = args[0][0] if isinstance(args[0], (tuple, list)) else args[0]
             x_out = out[0] if isinstance(out, (tuple, list)) else out
+            # a layer under activation checkpointing runs twice: first without a graph (nothing to hook), then again
+            # inside backward, where its output receives the gradient
             rec["x"][idx] = x_in.detach()
             rec["x"][idx + 1] = x_out.detach()
-            x_out.register_hook(lambda gr: rec["dy"].__setitem__(idx, gr.detach().clone()))
+            if x_out.requires_grad:
+                x_out.register_hook(lambda gr: rec["dy"].__setitem__(idx, gr.detach().clone()))
             if x_in.requires_grad:
                 x_in.register_hook(lambda gr: rec["dx"].__setitem__(idx, gr.detach().clone()))
         return fwd
@@ -73,6 +76,8 @@ def _hip_step(name, dev):
     for hk in hooks:
         hk.remove()
     out = dict(w=w, tokens=inputs[0], labels=labels, loss_mask=loss_mask, logits=logits_host, loss=loss.item(),
+               position_ids=inputs[1] if len(inputs) > 3 else None, cu_seqlens=inputs[3] if len(inputs) > 3 else None,
+               recomputed=model.recompute_count,
                grads={n: p.main_grad.cpu() for n, p in model.named_parameters()},
                W={k: v.detach().float().cpu() for k, v in model.state_dict().items() if "inv_freq" not in k},
                x={i: t.float().cpu() for i, t in rec["x"].items()},
@@ -88,7 +93,7 @@ def _layer_eval(r, cfg, i, storage):
     p = O.layer_prefix(i)
     Wl = {k: v.clone().requires_grad_(True) for k, v in r["W"].items() if k.startswith(p)}
     x = r["x"][i].clone().requires_grad_(True)
-    out = O.decoder_layer(x, Wl, p, cfg, storage_dtype=storage)
+    out = O.decoder_layer(x, Wl, p, cfg, position_ids=r["position_ids"], cu_seqlens=r["cu_seqlens"], storage_dtype=storage)
     out.backward(r["dy"][i])
     res = {"out": out.detach(), "dx": x.grad}
     res.update({k: v.grad for k, v in Wl.items()})
@@ -107,12 +112,12 @@ class _Lazy:
         return get
 
 
-def _layer_by_layer(name, r):
-    """Part 1 of the module docstring."""
+def _layer_by_layer(name, r, only=None):
+    """Part 1 of the module docstring.  only: the decoder layers to evaluate (default all)."""
     w, Wt, cfg = r["w"], r["W"], _oracle_cfg(r["w"])
     L = w["num_layers"]
     rep = P.Report(name)
-    for i in range(L):
+    for i in (range(L) if only is None else only):
         ref = _layer_eval(r, cfg, i, None)
         floor = _Lazy(lambda i=i: _layer_eval(r, cfg, i, torch.bfloat16))
         rep.check("layer %d output" % i, r["x"][i + 1], ref["out"], floor.item("out"))
@@ -137,7 +142,8 @@ def _layer_by_layer(name, r):
     ke = "1.word_embeddings.weight"
     ge = O.embedding_bwd(r["tokens"], r["dx"][0].transpose(0, 1), w["vocab_size"])
     rep.check("grad " + ke, r["grads"][ke], ge)
-    assert len([ln for ln in rep.lines if " grad " in ln]) == len(r["grads"])  # every parameter was compared
+    if only is None:
+        assert len([ln for ln in rep.lines if " grad " in ln]) == len(r["grads"])  # every parameter was compared
     return rep
 
 
@@ -163,6 +169,27 @@ def test_every_layer_of_the_full_size_step(gpu_device, name):
     assert all(" layer 0 " in ln or " grad 3." in ln for ln in rep.lines if "floor]" in ln)
 
 
+def test_first_and_last_layer_of_the_packed_workload(gpu_device):
+    """C5 at its own size (8 layers, 16384 packed tokens in 23 documents, position ids restarting per document, the first 4
+    layers recomputed in backward): decoder layers 0 (recomputed) and 7 (not), the final norm + head + loss and the embedding
+    gradient, each against the fp32 oracle evaluated from the HIP layer's own input and output gradient -- the packed
+    attention forward and backward at 32 heads and the per-document rotary positions at full size."""
+    name = "C5"
+    print("full-size parity, layers 0 and 7 + head, workload", name, flush=True)
+    r = _hip_step(name, gpu_device)
+    assert r["recomputed"] == 4 and r["cu_seqlens"] is not None and r["cu_seqlens"].numel() > 3
+    t0 = time.time()
+    rep = _layer_by_layer(name, r, only=(0, 7))
+    print("\n".join(rep.lines), flush=True)
+    print("%s: oracle, layers 0 and 7 + head: %.0f s on the host; %d of %d tensors at the bf16-storage floor, the rest at the "
+          "stated bar" % (name, time.time() - t0, rep.floor_used, len(rep.lines) - 1), flush=True)
+    assert not rep.failures, "\n".join(rep.failures)
+    assert all(" layer 0 " in ln or " grad 3." in ln for ln in rep.lines if "floor]" in ln)
+
+
+# Tensors of the end-to-end comparison that may use the floor rule: all of them -- the error of a four-layer chain of
+# bf16-stored ops is past the stated bar for the logits and for every gradient (the layer-by-layer test above is the gate
+# that holds each layer to the stated bar on identical inputs) -- but each within 5 % / 25 % of the floor.
 def test_headline_workload_end_to_end(gpu_device):
     name = "C2"
     print("full-size parity, end to end, workload", name, flush=True)

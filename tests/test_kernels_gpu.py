@@ -45,7 +45,8 @@ def K(gpu_device):
 
 
 # ------------------------------------------------------------------------------------- RMSNorm
-@pytest.mark.parametrize("rows,h", [(7, 256), (1024, 688), (515, 4096), (64, 8192), (3, 8)])
+@pytest.mark.parametrize("rows,h", [(7, 256), (1024, 688), (515, 4096), (64, 8192), (3, 8), (1537, 5120), (1030, 6144),
+                                    (2051, 8192), (5, 4104)])
 def test_rmsnorm_fwd_bwd(K, gpu_device, rows, h):
     print("rmsnorm", rows, h, flush=True)
     x, w, dy = rnd(rows, h, seed=1), (1 + 0.1 * torch.randn(h)).bfloat16(), rnd(rows, h, seed=2)
@@ -61,8 +62,8 @@ def test_rmsnorm_fwd_bwd(K, gpu_device, rows, h):
     close(mg, rdw + 1.0, "rmsnorm dw accumulate", rel=2e-3)
 
 
-def test_add_rmsnorm_fused(K, gpu_device):
-    rows, h = 130, 4096
+@pytest.mark.parametrize("rows,h", [(130, 4096), (1201, 8192), (77, 5120)])
+def test_add_rmsnorm_fused(K, gpu_device, rows, h):
     x, r, w = rnd(rows, h, seed=3), rnd(rows, h, seed=4), (1 + 0.1 * torch.randn(h)).bfloat16()
     y, rstd, s = K.rmsnorm_fwd(x.to(gpu_device), w.to(gpu_device), 1e-6, residual=r.to(gpu_device))
     ssum = (x.float() + r.float()).bfloat16()
@@ -189,6 +190,33 @@ def test_embedding_scatter_add_packed_batch_with_frequent_tokens(K, gpu_device):
     dW2 = torch.zeros(V, h, device=gpu_device)
     K.embed_scatter_add(ids.view(1, T).to(gpu_device), dy.view(1, T, h).to(gpu_device), dW2)
     assert torch.equal(dW2, dW)
+    # overwrite mode: whatever the buffer held is gone, ids that do not occur get zero rows
+    dW3 = torch.full((V, h), 3.5, device=gpu_device)
+    K.embed_scatter_add(ids.view(1, T).to(gpu_device), dy.view(1, T, h).to(gpu_device), dW3, accumulate=False)
+    assert torch.equal(dW3, dW)
+
+
+def test_embedding_scatter_add_with_an_id_that_fills_most_of_a_long_batch(K, gpu_device):
+    """20000 rows of which 11000 carry one id (a padding token): more than one 8192-row window of the ordering bitmap, and
+    more rows of one id than a window holds.  Row-order fp32 sums, bit for bit, in both modes."""
+    T, V, h = 20000, 1000, 264
+    g = torch.Generator().manual_seed(6)
+    ids = torch.randint(0, V, (T,), generator=g)
+    ids[torch.randperm(T, generator=g)[:11000]] = 999
+    ids[torch.randperm(T, generator=g)[:1500]] = 0
+    dy = rnd(T, h, seed=12)
+    print("embed scatter, frequent id", flush=True)
+    seq = torch.zeros(V, h)
+    dyf = dy.float()
+    for r, i in enumerate(ids.tolist()):
+        seq[i] += dyf[r]
+    dW = torch.full((V, h), -1.25, device=gpu_device)
+    K.embed_scatter_add(ids.view(1, T).to(gpu_device), dy.view(1, T, h).to(gpu_device), dW, accumulate=False)
+    assert torch.equal(dW.cpu(), seq)
+    init = torch.randn(V, h, generator=g)
+    dW = init.to(gpu_device)
+    K.embed_scatter_add(ids.view(1, T).to(gpu_device), dy.view(1, T, h).to(gpu_device), dW)
+    assert torch.equal(dW.cpu(), init + seq)
 
 
 # ------------------------------------------------------------------------------------- plumbing
