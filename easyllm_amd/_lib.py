@@ -35,7 +35,7 @@ SIGNATURES = {
     "ezl_gemm_bf16_ksplit": [_i32, _vpp, _vpp, _vp, _i64, _i64, _i64p, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
     "ezl_attn_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64p, _vp],
     "ezl_attn_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32,
-                     _i64p, _vp],
+                     _i64p, _vp, _i64, _vp],
     "ezl_mask_compact": [_vp, _i64, _i64, _vp, _vp, _vp, _vp],
     "ezl_rows_gather": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     "ezl_ce_prepare": [_vp, _vp, _i32, _i64, _vp, _vp, _i64, _vp],
@@ -56,6 +56,7 @@ _SPECIAL = {
     "ezl_rmsnorm_bwd_noalloc_max_h": ([], _i64),
     "ezl_bias_grad_workspace_bytes": ([_i64, _i64], _i64),
     "ezl_embed_scatter_add_workspace_bytes": ([_i64, _i64], _i64),
+    "ezl_attn_bwd_workspace_bytes": ([_i64, _i64, _i64, _i64, _i64], _i64),
     "ezl_sumsq_partials": ([], _i64),
     "ezl_location_idx_rows": ([_i64, _i64, _i64], _i64),
 }
@@ -107,6 +108,10 @@ def bias_grad_workspace_bytes(rows, n):
 
 def embed_scatter_add_workspace_bytes(rows, vocab):
     return load().ezl_embed_scatter_add_workspace_bytes(rows, vocab)
+
+
+def attn_bwd_workspace_bytes(total_tokens, ndocs, nq, nk, d):
+    return load().ezl_attn_bwd_workspace_bytes(total_tokens, ndocs, nq, nk, d)
 
 
 def sumsq_partials():

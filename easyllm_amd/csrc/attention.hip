@@ -27,6 +27,9 @@
 namespace {
 
 constexpr int kThreads = 256;
+#ifndef EZL_DKDV_MIN_BLOCKS
+#define EZL_DKDV_MIN_BLOCKS 512  // dK/dV workgroups wanted before (kv head, key block) pairs stop being split
+#endif
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -38,6 +41,8 @@ struct AttnParams {
     const bf16_t* q; const bf16_t* k; const bf16_t* v; const bf16_t* o; const bf16_t* dout;
     bf16_t* out; bf16_t* dq; bf16_t* dk; bf16_t* dv;
     float* lse; float* delta;
+    float* part;  // dK/dV kernel with nsplit > 1: fp32 partial sums [nsplit][2 (dK, dV)][T][nk][d]
+    int nsplit;   // workgroups that share a (kv head, key block): each takes nq / nk / nsplit of the group's query heads
     const int* cu;
     int ndocs, s_len, T, nq, nk;
     float scale;
@@ -547,29 +552,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
 }
 
 // =================================================================================================
-// delta[h, n] = sum_d dO[n, h, d] * O[n, h, d]
-// =================================================================================================
-template <int D>
-__global__ __launch_bounds__(kThreads) void attn_delta_kernel(AttnParams p) {
-    constexpr int TPR = D / 8;  // threads per (token, head)
-    const int64_t items = (int64_t)p.T * p.nq;
-    const int sub = threadIdx.x % TPR;
-    // a (token, head) pair is owned by TPR consecutive lanes, which enter and leave the loop together
-    for (int64_t it = ((int64_t)blockIdx.x * kThreads + threadIdx.x) / TPR; it < items;
-         it += (int64_t)gridDim.x * (kThreads / TPR)) {
-        const int n = (int)(it / p.nq), h = (int)(it % p.nq);
-        float a[8], b[8], acc = 0.f;
-        unpack8(ld_bf16x8(p.o + tok_off(n, p.s_len, p.o_ss, p.o_sb) + (int64_t)h * D + sub * 8), a);
-        unpack8(ld_bf16x8(p.dout + tok_off(n, p.s_len, p.do_ss, p.do_sb) + (int64_t)h * D + sub * 8), b);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc += a[i] * b[i];
-#pragma unroll
-        for (int o = TPR / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-        if (sub == 0) p.delta[(int64_t)h * p.T + n] = acc;
-    }
-}
-
-// =================================================================================================
 // backward, dK and dV: a block owns 128 keys of one kv head and walks the queries at or after them
 // =================================================================================================
 // 8 waves: wave w works on keys 32 (w & 3) .. +31 and, of every 64-query tile, on the 32-query half (w >> 2); the two
@@ -591,12 +573,15 @@ __global__ __launch_bounds__(kDkdvThreads) void attn_bwd_dkdv_kernel(AttnParams 
                   "the final reduction parks four waves' accumulators in the tile memory");
     int doc_start, doc_len, kbk;
     int bx, by;
-    xcd_head_blocks(p.nk, bx, by);
+    xcd_head_blocks(p.nk * p.nsplit, bx, by);
     if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, kbk)) return;
     kbk = (doc_len + 127) / 128 - 1 - kbk;  // rank 0 = most blocks of queries to walk = the piece's first keys
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kg = wave & 3, half = wave >> 2;
-    const int hk = by, group = p.nq / p.nk;
+    // With a large GQA group a (kv head, key block) is long and there are few of them: the group's query heads are dealt
+    // to nsplit workgroups, each leaving fp32 partial sums that attn_dkdv_combine_kernel adds in a fixed order.
+    const int hk = by / p.nsplit, part = by - hk * p.nsplit;
+    const int group = p.nq / p.nk / p.nsplit, hq0 = hk * (p.nq / p.nk) + part * group;
     const int k0 = kbk * 128, kw0 = k0 + kg * 32;
     const int tok_end = doc_start + doc_len;
     const int kj = kw0 + (lane & 31);  // this lane's key (document relative)
@@ -640,7 +625,7 @@ __global__ __launch_bounds__(kDkdvThreads) void attn_bwd_dkdv_kernel(AttnParams 
     bf16x8 rq[NCH_Q], rdo[NCH_Q];
     float rstat = 0.f;  // threads 0..63: lse*log2e of query tid; 64..127: delta of query tid-64
     auto load_iter = [&](int it) {
-        const int hq = hk * group + it / nqt;
+        const int hq = hq0 + it / nqt;
         const int row0 = (qt0 + it % nqt) * 64;
 #pragma unroll
         for (int i = 0; i < NCH_Q; ++i) {
@@ -717,22 +702,29 @@ __global__ __launch_bounds__(kDkdvThreads) void attn_bwd_dkdv_kernel(AttnParams 
                 }
             };
             ldt(0, 0);
-            // accumulator register r <-> query qs0 + acc_row(r); lane <-> key kj
+            // accumulator register r <-> query qs0 + acc_row(r); lane <-> key kj.  Only a tile that meets the diagonal of this
+            // wave's keys or the document's end needs the mask (a wave-uniform property).
+            auto probabilities = [&](auto MASKED) {
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const int ql = half * 32 + 8 * r4 + 4 * (lane >> 5);
-                const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sstat[cur][0][ql]);
-                const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sstat[cur][1][ql]);
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    const int ql = half * 32 + 8 * r4 + 4 * (lane >> 5);
+                    const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sstat[cur][0][ql]);
+                    const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sstat[cur][1][ql]);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int r = r4 * 4 + e;
-                    const int qidx = qbase + ql + e;
-                    float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], sl2, -l4[e]));
-                    if (kj > qidx || qidx >= doc_len) pe = 0.f;
-                    sacc[r] = pe;
-                    dpacc[r] = pe * (dpacc[r] - d4[e]);
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = r4 * 4 + e;
+                        float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], sl2, -l4[e]));
+                        if constexpr (decltype(MASKED)::value) {
+                            const int qidx = qbase + ql + e;
+                            if (kj > qidx || qidx >= doc_len) pe = 0.f;
+                        }
+                        sacc[r] = pe;
+                        dpacc[r] = pe * (dpacc[r] - d4[e]);
+                    }
                 }
-            }
+            };
+            if (qs0 < kw0 + 31 || qs0 + 32 > doc_len) probabilities(std::true_type{});
+            else probabilities(std::false_type{});
 #pragma unroll
             for (int gt = 0; gt < NT; ++gt) {
                 if (gt + 1 < NT) ldt(gt + 1, (gt + 1) & 1);
@@ -763,6 +755,27 @@ __global__ __launch_bounds__(kDkdvThreads) void attn_bwd_dkdv_kernel(AttnParams 
     }
     __syncthreads();
     if (half == 0 && kj < doc_len) {
+        if (p.nsplit > 1) {  // fp32 partial sums of this workgroup's query heads, unscaled
+            const int64_t slab = (int64_t)p.T * p.nk * D;
+            float* pk = p.part + (int64_t)part * 2 * slab + ((int64_t)(doc_start + kj) * p.nk + hk) * D;
+            float* pv = pk + slab;
+#pragma unroll
+            for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    f32x4 a, b;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int r = r4 * 4 + e;
+                        a[e] = dkacc[db][r] + red[(db * 16 + r) * 64 + lane];
+                        b[e] = dvacc[db][r] + red[((D / 32 + db) * 16 + r) * 64 + lane];
+                    }
+                    const int dcol = db * 32 + 8 * r4 + 4 * (lane >> 5);
+                    *reinterpret_cast<f32x4*>(pk + dcol) = a;
+                    *reinterpret_cast<f32x4*>(pv + dcol) = b;
+                }
+            return;
+        }
         bf16_t* dkrow = p.dk + tok_off(doc_start + kj, p.s_len, p.dk_ss, p.dk_sb) + (int64_t)hk * D;
         bf16_t* dvrow = p.dv + tok_off(doc_start + kj, p.s_len, p.dv_ss, p.dv_sb) + (int64_t)hk * D;
 #pragma unroll
@@ -780,6 +793,34 @@ __global__ __launch_bounds__(kDkdvThreads) void attn_bwd_dkdv_kernel(AttnParams 
                 *reinterpret_cast<bf16x4*>(dkrow + dcol) = a;
                 *reinterpret_cast<bf16x4*>(dvrow + dcol) = b;
             }
+    }
+}
+
+// dK = scale * sum_parts partial dK, dV = sum_parts partial dV, parts added in index order; one thread per 8 columns
+template <int D>
+__global__ __launch_bounds__(kThreads) void attn_dkdv_combine_kernel(AttnParams p) {
+    const int64_t slab = (int64_t)p.T * p.nk * D;
+    const int64_t chunks = slab / 8;
+    for (int64_t c = (int64_t)blockIdx.x * kThreads + threadIdx.x; c < chunks; c += (int64_t)gridDim.x * kThreads) {
+        const int64_t e0 = c * 8;
+        const int n = (int)(e0 / ((int64_t)p.nk * D));
+        const int rem = (int)(e0 - (int64_t)n * p.nk * D);  // head * D + column
+        float k8[8], v8[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { k8[i] = 0.f; v8[i] = 0.f; }
+        for (int s = 0; s < p.nsplit; ++s) {
+            const float* pk = p.part + (int64_t)s * 2 * slab + e0;
+            const f32x4 a0 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pk));
+            const f32x4 a1 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pk + 4));
+            const f32x4 b0 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pk + slab));
+            const f32x4 b1 = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pk + slab + 4));
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { k8[i] += a0[i]; k8[4 + i] += a1[i]; v8[i] += b0[i]; v8[4 + i] += b1[i]; }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) k8[i] *= p.scale;
+        st_bf16x8(p.dk + tok_off(n, p.s_len, p.dk_ss, p.dk_sb) + rem, pack8(k8));
+        st_bf16x8(p.dv + tok_off(n, p.s_len, p.dv_ss, p.dv_sb) + rem, pack8(v8));
     }
 }
 
@@ -804,7 +845,20 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
     load_row_frags<D>(p.q + tok_off(qtok, p.s_len, p.q_ss, p.q_sb) + (int64_t)hq * D, lane, qf);
     load_row_frags<D>(p.dout + tok_off(qtok, p.s_len, p.do_ss, p.do_sb) + (int64_t)hq * D, lane, dof);
     const float lse2 = p.lse[(int64_t)hq * p.T + qtok] * kLog2e;
-    const float dlt = p.delta[(int64_t)hq * p.T + qtok];
+    // delta = sum_d dO * O of this lane's query: the lane holds one half of the row's columns, its partner (lane ^ 32) the
+    // other.  Written out for the dK/dV kernel, which runs after this one.
+    float dlt = 0.f;
+    {
+        const bf16_t* orow = p.o + tok_off(qtok, p.s_len, p.o_ss, p.o_sb) + (int64_t)hq * D;
+#pragma unroll
+        for (int kd = 0; kd < D / 16; ++kd) {
+            const bf16x8 ov = *reinterpret_cast<const bf16x8*>(orow + kd * 16 + (lane >> 5) * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dlt += (float)ov[e] * (float)dof[kd][e];
+        }
+        dlt += __shfl_xor(dlt, 32, 64);
+        if (lane < 32 && qi < doc_len) p.delta[(int64_t)hq * p.T + doc_start + qi] = dlt;
+    }
 
     const int kend = (q0 + 128 < doc_len ? q0 + 128 : doc_len);
     const int ntiles = (kend + 63) / 64;
@@ -956,10 +1010,30 @@ extern "C" int ezl_attn_fwd(const void* q, const void* k, const void* v, void* o
     return EZL_OK;
 }
 
+namespace {
+// workgroups per (kv head, key block) of the dK/dV kernel: enough of them for two rounds of the 256 CUs, so that a long
+// block from the start of a document and a short one from its end share a CU (measured at 64 q / 8 kv heads, s = 4096:
+// 1080 us unsplit, 582 us with 2 parts, 578 us with 4 parts, whose partial sums cost twice as much to add)
+int attn_bwd_split(int64_t total_tokens, int64_t ndocs, int64_t nq, int64_t nk) {
+    const int64_t group = nq / nk;
+    const int64_t blocks = nk * ((total_tokens + 127) / 128 + ndocs - 1);
+    int split = 1;
+    while (blocks * split < EZL_DKDV_MIN_BLOCKS && group % (split * 2) == 0) split *= 2;
+    return split;
+}
+}  // namespace
+
+extern "C" int64_t ezl_attn_bwd_workspace_bytes(int64_t total_tokens, int64_t ndocs, int64_t nq, int64_t nk, int64_t d) {
+    if (total_tokens < 0 || ndocs <= 0 || nq <= 0 || nk <= 0 || nq % nk != 0 || d <= 0) return -1;
+    const int split = attn_bwd_split(total_tokens, ndocs, nq, nk);
+    return split > 1 ? (int64_t)split * 2 * total_tokens * nk * d * (int64_t)sizeof(float) : 0;
+}
+
 // strides[16]: q, k, v, out (as above), then dout, dq, dk, dv (seq, batch each)
 extern "C" int ezl_attn_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout, const void* lse,
                             void* delta, void* dq, void* dk, void* dv, const void* cu_seqlens, int64_t ndocs, int64_t total_tokens,
-                            int64_t s_len, int64_t nq, int64_t nk, int64_t d, float scale, const int64_t* strides, void* stream) {
+                            int64_t s_len, int64_t nq, int64_t nk, int64_t d, float scale, const int64_t* strides, void* workspace,
+                            int64_t workspace_bytes, void* stream) {
     int rc = check_common("ezl_attn_bwd", total_tokens, s_len, nq, nk, d, ndocs, strides, 16);
     if (rc) return rc;
     if (total_tokens == 0) return EZL_OK;
@@ -967,30 +1041,35 @@ extern "C" int ezl_attn_bwd(const void* q, const void* k, const void* v, const v
     EZL_REQUIRE(ezl_aligned16(q) && ezl_aligned16(k) && ezl_aligned16(v) && ezl_aligned16(out) && ezl_aligned16(dout) &&
                     ezl_aligned16(dq) && ezl_aligned16(dk) && ezl_aligned16(dv),
                 EZL_EINVAL, "ezl_attn_bwd: misaligned pointer");
+    const int64_t need = ezl_attn_bwd_workspace_bytes(total_tokens, ndocs, nq, nk, d);
+    EZL_REQUIRE(need == 0 || (workspace && ezl_aligned16(workspace) && workspace_bytes >= need), EZL_EINVAL,
+                "ezl_attn_bwd: workspace missing, misaligned or smaller than ezl_attn_bwd_workspace_bytes()");
     AttnParams p = {};
     p.q = (const bf16_t*)q; p.k = (const bf16_t*)k; p.v = (const bf16_t*)v; p.o = (const bf16_t*)out; p.dout = (const bf16_t*)dout;
     p.lse = (float*)const_cast<void*>(lse); p.delta = (float*)delta; p.dq = (bf16_t*)dq; p.dk = (bf16_t*)dk; p.dv = (bf16_t*)dv;
     p.cu = (const int*)cu_seqlens; p.ndocs = (int)ndocs; p.s_len = (int)s_len; p.T = (int)total_tokens; p.nq = (int)nq; p.nk = (int)nk;
     p.scale = scale;
+    p.nsplit = attn_bwd_split(total_tokens, ndocs, nq, nk);
+    p.part = p.nsplit > 1 ? (float*)workspace : nullptr;
     p.q_ss = strides[0]; p.q_sb = strides[1]; p.k_ss = strides[2]; p.k_sb = strides[3];
     p.v_ss = strides[4]; p.v_sb = strides[5]; p.o_ss = strides[6]; p.o_sb = strides[7];
     p.do_ss = strides[8]; p.do_sb = strides[9]; p.dq_ss = strides[10]; p.dq_sb = strides[11];
     p.dk_ss = strides[12]; p.dk_sb = strides[13]; p.dv_ss = strides[14]; p.dv_sb = strides[15];
     hipStream_t st = (hipStream_t)stream;
-    const int64_t items = total_tokens * nq;
-    const int per_block = kThreads / (int)(d / 8);
-    int64_t g = (items + per_block - 1) / per_block;
-    if (g > 256 * 32) g = 256 * 32;
-    const dim3 gridq((unsigned)((total_tokens + 127) / 128 + ndocs + total_tokens / s_len), (unsigned)nq);
-    const dim3 gridk((unsigned)((total_tokens + 127) / 128 + ndocs + total_tokens / s_len), (unsigned)nk);
+    const unsigned nblk = (unsigned)((total_tokens + 127) / 128 + ndocs + total_tokens / s_len);
+    const dim3 gridq(nblk, (unsigned)nq);
+    const dim3 gridk(nblk, (unsigned)(nk * p.nsplit));
+    int64_t gc = (total_tokens * nk * d / 8 + kThreads - 1) / kThreads;
+    if (gc > 256 * 16) gc = 256 * 16;
+    // the dQ kernel goes first: it also produces delta = rowsum(dO * O), which the dK/dV kernel reads
     if (d == 128) {
-        hipLaunchKernelGGL(attn_delta_kernel<128>, dim3((unsigned)g), dim3(kThreads), 0, st, p);
-        hipLaunchKernelGGL(attn_bwd_dkdv_kernel<128>, gridk, dim3(kDkdvThreads), 0, st, p);
         hipLaunchKernelGGL(attn_bwd_dq_kernel<128>, gridq, dim3(kThreads), 0, st, p);
+        hipLaunchKernelGGL(attn_bwd_dkdv_kernel<128>, gridk, dim3(kDkdvThreads), 0, st, p);
+        if (p.nsplit > 1) hipLaunchKernelGGL(attn_dkdv_combine_kernel<128>, dim3((unsigned)gc), dim3(kThreads), 0, st, p);
     } else {
-        hipLaunchKernelGGL(attn_delta_kernel<64>, dim3((unsigned)g), dim3(kThreads), 0, st, p);
-        hipLaunchKernelGGL(attn_bwd_dkdv_kernel<64>, gridk, dim3(kDkdvThreads), 0, st, p);
         hipLaunchKernelGGL(attn_bwd_dq_kernel<64>, gridq, dim3(kThreads), 0, st, p);
+        hipLaunchKernelGGL(attn_bwd_dkdv_kernel<64>, gridk, dim3(kDkdvThreads), 0, st, p);
+        if (p.nsplit > 1) hipLaunchKernelGGL(attn_dkdv_combine_kernel<64>, dim3((unsigned)gc), dim3(kThreads), 0, st, p);
     }
     EZL_LAUNCH_CHECK("ezl_attn_bwd");
     return EZL_OK;

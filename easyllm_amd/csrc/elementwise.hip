@@ -136,7 +136,8 @@ __global__ __launch_bounds__(kBlock) void ids_in_range_kernel(const int64_t* __r
 }
 
 // out[r, :] = W[ids[r], :]; an id outside [0, V) raises the flag and yields a zero row.
-// One wave per row; a lane's loads (up to 4 vectors of 8 at a time) are all in flight before its first store.
+// One wave per row; a lane's loads (up to 8 vectors of 8 at a time: a row of 4096 in one go) are all in flight before its
+// first store.
 __global__ __launch_bounds__(kBlock) void embed_gather_kernel(const int64_t* __restrict__ ids, const bf16_t* __restrict__ W,
                                                               bf16_t* __restrict__ out, int64_t rows, int h, int64_t V,
                                                               int* __restrict__ bad_flag) {
@@ -148,16 +149,16 @@ __global__ __launch_bounds__(kBlock) void embed_gather_kernel(const int64_t* __r
         if (!ok && lane == 0) atomicOr(bad_flag, id >= V ? 1 : 2);
         const bf16_t* src = W + (ok ? id : 0) * h;
         bf16_t* dst = out + r * h;
-        for (int c0 = lane; c0 < h8; c0 += 256) {
-            bf16x8 v[4];
+        for (int c0 = lane; c0 < h8; c0 += 512) {
+            bf16x8 v[8];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < 8; ++u) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k) v[u][k] = (bf16_t)0.0f;
                 if (ok && c0 + u * 64 < h8) v[u] = ld_bf16x8(src + (c0 + u * 64) * 8);
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
+            for (int u = 0; u < 8; ++u)
                 if (c0 + u * 64 < h8) st_bf16x8(dst + (c0 + u * 64) * 8, v[u]);
         }
     }
@@ -381,12 +382,22 @@ __global__ __launch_bounds__(kBlock) void embed_scatter_bucket_kernel(const int6
             }
         }
     }
-    if (overwrite) {  // ids that do not occur: zero rows
+    if (overwrite) {
+        // ids that do not occur: zero rows.  A block takes a contiguous range of the vocabulary and reads the counts of up
+        // to kBlock rows at once, so that the fill streams instead of waiting for one count per row.
         const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-        for (int64_t v = blockIdx.x; v < V; v += gridDim.x) {
-            if (cnt[v] != 0) continue;
-            float* dst = dW + v * h;
-            for (int i = threadIdx.x; i < (h >> 2); i += kBlock) __builtin_nontemporal_store(z, reinterpret_cast<f32x4*>(dst) + i);
+        const int64_t per = (V + gridDim.x - 1) / gridDim.x;
+        const int64_t vbeg = (int64_t)blockIdx.x * per, vend = vbeg + per < V ? vbeg + per : V;
+        for (int64_t v0 = vbeg; v0 < vend; v0 += kBlock) {
+            const int m = vend - v0 < kBlock ? (int)(vend - v0) : kBlock;
+            __syncthreads();
+            if ((int)threadIdx.x < m) raw[threadIdx.x] = cnt[v0 + threadIdx.x];
+            __syncthreads();
+            for (int r = 0; r < m; ++r) {
+                if (raw[r] != 0) continue;
+                f32x4* dst = reinterpret_cast<f32x4*>(dW + (v0 + r) * h);
+                for (int i = threadIdx.x; i < (h >> 2); i += kBlock) dst[i] = z;
+            }
         }
     }
 }

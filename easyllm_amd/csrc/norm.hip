@@ -5,9 +5,9 @@
 // of llama/transformer.py:786 fused in front (sum rounded to bf16 first, as the reference's bf16
 // tensor add does).
 //
-// Layout: rows of h bf16, h % 8 == 0, h <= 8192.  A row is held in registers (read from HBM exactly once): forward by
+// Layout: rows of h bf16, h % 8 == 0.  Up to h = 8192 a row is held in registers (read from HBM exactly once): forward by
 // TPR = min(256, h/8 rounded up to a wave) threads whose row sums meet through a double-buffered LDS cell; backward by one
-// wave (h <= 4096) or by a pair of waves (wider rows).
+// wave (h <= 4096) or by a pair of waves (wider rows).  Rows up to 32768 wide go through two-pass kernels.
 #include "common.h"
 
 #include <mutex>
@@ -258,6 +258,116 @@ __global__ __launch_bounds__(256, 2) void rmsnorm_bwd_pair_kernel(const bf16_t* 
     for (int j = threadIdx.x; j < h; j += 256) dw_partial[(size_t)blockIdx.x * h + j] = fold[j];
 }
 
+// ---- rows wider than 8192 (up to kWideMaxH) --------------------------------------------------------------------------
+// The reference leaves such rows to its unfused path (fused_layer_norm.py:56, :68-71).  Here a block of 1024 threads walks a
+// row twice -- once for the row statistic, once to produce the output (the second read comes from cache) -- so nothing
+// depends on the row fitting into registers.  Backward keeps the dw column sums of the block's rows in LDS, every thread
+// adding only to its own columns (no atomics, fixed order), and writes one partial row per block.
+constexpr int kWideMaxH = 32768;
+constexpr int kWideThreads = 1024;
+
+__device__ __forceinline__ float block_sum_1024(float v, float (*red)[kWideThreads / 64], int& parity) {
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[parity][threadIdx.x >> 6] = v;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < kWideThreads / 64; ++i) t += red[parity][i];
+    parity ^= 1;  // the next sum uses the other set of cells: one barrier per sum
+    return t;
+}
+
+template <bool HAS_RES>
+__global__ __launch_bounds__(kWideThreads) void rmsnorm_fwd_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ res,
+                                                                        const bf16_t* __restrict__ w, bf16_t* __restrict__ y,
+                                                                        bf16_t* __restrict__ sum_out, float* __restrict__ rstd_out,
+                                                                        int T, int h, float eps) {
+    __shared__ float red[2][kWideThreads / 64];
+    const int h8 = h >> 3;
+    int parity = 0;
+    for (int row = blockIdx.x; row < T; row += gridDim.x) {
+        const size_t base = (size_t)row * h;
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < h8; c += kWideThreads) {
+            float v[8];
+            unpack8(ld_bf16x8(x + base + c * 8), v);
+            if (HAS_RES) {
+                float r[8];
+                unpack8(ld_bf16x8(res + base + c * 8), r);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = (float)(bf16_t)(v[i] + r[i]);
+                st_bf16x8(sum_out + base + c * 8, pack8(v));
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
+        }
+        ss = block_sum_1024(ss, red, parity);
+        const float rs = rsqrtf(ss / (float)h + eps);
+        if (threadIdx.x == 0) rstd_out[row] = rs;
+        for (int c = threadIdx.x; c < h8; c += kWideThreads) {
+            float v[8], wv[8], o[8];
+            unpack8(ld_bf16x8(x + base + c * 8), v);
+            if (HAS_RES) {  // recomputed rather than read back from sum_out
+                float r[8];
+                unpack8(ld_bf16x8(res + base + c * 8), r);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = (float)(bf16_t)(v[i] + r[i]);
+            }
+            unpack8(ld_bf16x8(w + c * 8), wv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = v[i] * rs * wv[i];
+            st_bf16x8(y + base + c * 8, pack8(o));
+        }
+    }
+}
+
+template <bool HAS_DRES>
+__global__ __launch_bounds__(kWideThreads) void rmsnorm_bwd_wide_kernel(const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
+                                                                        const bf16_t* __restrict__ w, const float* __restrict__ rstd,
+                                                                        const bf16_t* __restrict__ dres, bf16_t* __restrict__ dx,
+                                                                        float* __restrict__ dw_partial, int T, int h) {
+    __shared__ float fold[kWideMaxH];  // dw sums over this block's rows; thread t owns columns 8 (c * 1024 + t) .. + 7
+    __shared__ float red[2][kWideThreads / 64];
+    const int h8 = h >> 3;
+    for (int c = threadIdx.x; c < h8; c += kWideThreads)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) fold[c * 8 + i] = 0.f;
+    int parity = 0;
+    const float inv_h = 1.0f / (float)h;
+    for (int row = blockIdx.x; row < T; row += gridDim.x) {
+        const size_t base = (size_t)row * h;
+        const float rs = rstd[row];
+        float dot = 0.f;
+        for (int c = threadIdx.x; c < h8; c += kWideThreads) {
+            float xv[8], dyv[8], wv[8];
+            unpack8(ld_bf16x8(x + base + c * 8), xv);
+            unpack8(ld_bf16x8(dy + base + c * 8), dyv);
+            unpack8(ld_bf16x8(w + c * 8), wv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dot += dyv[i] * wv[i] * (xv[i] * rs);
+        }
+        const float cmean = block_sum_1024(dot, red, parity) * inv_h;
+        for (int c = threadIdx.x; c < h8; c += kWideThreads) {
+            float xv[8], dyv[8], wv[8], o[8];
+            unpack8(ld_bf16x8(x + base + c * 8), xv);
+            unpack8(ld_bf16x8(dy + base + c * 8), dyv);
+            unpack8(ld_bf16x8(w + c * 8), wv);
+            if (HAS_DRES) unpack8(ld_bf16x8(dres + base + c * 8), o);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float xhat = xv[i] * rs;
+                const float g = rs * (dyv[i] * wv[i] - xhat * cmean);
+                o[i] = HAS_DRES ? o[i] + g : g;
+                fold[c * 8 + i] += dyv[i] * xhat;
+            }
+            st_bf16x8(dx + base + c * 8, pack8(o));
+        }
+    }
+    for (int c = threadIdx.x; c < h8; c += kWideThreads)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dw_partial[(size_t)blockIdx.x * h + c * 8 + i] = fold[c * 8 + i];
+}
+
 int tpr_for(int h) {
     int t = (h / 8 + 63) / 64 * 64;
     return t < 64 ? 64 : (t > 256 ? 256 : t);
@@ -267,8 +377,8 @@ int tpr_for(int h) {
 
 extern "C" int ezl_rmsnorm_fwd(const void* x, const void* residual, const void* weight, void* y, void* sum_out,
                                void* rstd, int64_t rows, int64_t h, float eps, void* stream) {
-    EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h <= 8192, EZL_EUNSUPPORTED,
-                "ezl_rmsnorm_fwd: need h %% 8 == 0 and h <= 8192 (got h=%lld)", (long long)h);
+    EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h <= kWideMaxH, EZL_EUNSUPPORTED,
+                "ezl_rmsnorm_fwd: need h %% 8 == 0 and h <= %d (got h=%lld)", kWideMaxH, (long long)h);
     EZL_REQUIRE(rows == 0 || (x && weight && y && rstd), EZL_EINVAL, "ezl_rmsnorm_fwd: null pointer");
     EZL_REQUIRE((residual == nullptr) == (sum_out == nullptr), EZL_EINVAL,
                 "ezl_rmsnorm_fwd: residual and sum_out go together");
@@ -276,17 +386,28 @@ extern "C" int ezl_rmsnorm_fwd(const void* x, const void* residual, const void* 
                     ezl_aligned16(sum_out),
                 EZL_EINVAL, "ezl_rmsnorm_fwd: pointers must be 16-byte aligned");
     if (rows == 0) return EZL_OK;
+    hipStream_t st = (hipStream_t)stream;
+    EZL_REQUIRE(rows < (1LL << 31), EZL_EUNSUPPORTED, "ezl_rmsnorm_fwd: too many rows");
+    if (h > 8192) {
+        const unsigned g = (unsigned)(rows < 512 ? rows : 512);
+        if (residual)
+            hipLaunchKernelGGL(rmsnorm_fwd_wide_kernel<true>, dim3(g), dim3(kWideThreads), 0, st, (const bf16_t*)x, (const bf16_t*)residual,
+                               (const bf16_t*)weight, (bf16_t*)y, (bf16_t*)sum_out, (float*)rstd, (int)rows, (int)h, eps);
+        else
+            hipLaunchKernelGGL(rmsnorm_fwd_wide_kernel<false>, dim3(g), dim3(kWideThreads), 0, st, (const bf16_t*)x, (const bf16_t*)residual,
+                               (const bf16_t*)weight, (bf16_t*)y, (bf16_t*)sum_out, (float*)rstd, (int)rows, (int)h, eps);
+        EZL_LAUNCH_CHECK("ezl_rmsnorm_fwd");
+        return EZL_OK;
+    }
     const int tpr = tpr_for((int)h);
     const int nchunk = ((int)h + tpr * 8 - 1) / (tpr * 8);
     const int rpb = 256 / tpr;
     int64_t grid = (rows + rpb - 1) / rpb;
     if (grid > 256 * 16) grid = 256 * 16;
-    hipStream_t st = (hipStream_t)stream;
 #define LAUNCH(NC, RES)                                                                                             \
     hipLaunchKernelGGL((rmsnorm_fwd_kernel<NC, RES>), dim3((unsigned)grid), dim3(256), 0, st, (const bf16_t*)x,      \
                        (const bf16_t*)residual, (const bf16_t*)weight, (bf16_t*)y, (bf16_t*)sum_out, (float*)rstd, \
                        (int)rows, (int)h, eps, tpr)
-    EZL_REQUIRE(rows < (1LL << 31), EZL_EUNSUPPORTED, "ezl_rmsnorm_fwd: too many rows");
     if (residual) {
         if (nchunk == 1) LAUNCH(1, true); else if (nchunk == 2) LAUNCH(2, true); else LAUNCH(4, true);
     } else {
@@ -299,7 +420,7 @@ extern "C" int ezl_rmsnorm_fwd(const void* x, const void* residual, const void* 
 
 namespace {
 // blocks (= fp32 partial rows of h) the backward kernels want: 8 waves per CU in both forms
-int64_t rmsnorm_bwd_blocks(int64_t h) { return h <= 4096 ? 256 : 512; }
+int64_t rmsnorm_bwd_blocks(int64_t h) { return h <= 4096 ? 256 : (h <= 8192 ? 512 : 256); }
 }  // namespace
 
 extern "C" int64_t ezl_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t h) {
@@ -311,8 +432,8 @@ namespace {
 
 int rmsnorm_bwd_check(const char* name, const void* dy, const void* x, const void* weight, const void* rstd, const void* dresidual,
                       const void* dx, const void* dw_bf16, const void* dw_f32, int64_t rows, int64_t h) {
-    EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h <= 8192, EZL_EUNSUPPORTED, "%s: need h %% 8 == 0 and h <= 8192 (got h=%lld)",
-                name, (long long)h);
+    EZL_REQUIRE(rows >= 0 && h > 0 && h % 8 == 0 && h <= kWideMaxH, EZL_EUNSUPPORTED, "%s: need h %% 8 == 0 and h <= %d (got h=%lld)",
+                name, kWideMaxH, (long long)h);
     EZL_REQUIRE(weight && (rows == 0 || (dy && x && rstd && dx)), EZL_EINVAL, "%s: null pointer", name);
     EZL_REQUIRE((dw_bf16 != nullptr) != (dw_f32 != nullptr), EZL_EINVAL, "%s: exactly one of dw_bf16 / dw_f32", name);
     EZL_REQUIRE(ezl_aligned16(dy) && ezl_aligned16(x) && ezl_aligned16(weight) && ezl_aligned16(dx) && ezl_aligned16(dresidual),
@@ -347,6 +468,15 @@ int rmsnorm_bwd_launch(const void* dy, const void* x, const void* weight, const 
         if (dresidual) LAUNCH_NC(true); else LAUNCH_NC(false);
 #undef LAUNCH_NC
 #undef LAUNCH
+    } else if (h > 8192) {  // rows that do not fit into registers: two passes per row, dw sums in LDS
+        grid = rows < max_blocks ? rows : max_blocks;
+        if (grid < 1) grid = 1;
+        if (dresidual)
+            hipLaunchKernelGGL(rmsnorm_bwd_wide_kernel<true>, dim3((unsigned)grid), dim3(kWideThreads), 0, st, (const bf16_t*)dy, (const bf16_t*)x,
+                               (const bf16_t*)weight, (const float*)rstd, (const bf16_t*)dresidual, (bf16_t*)dx, partials, (int)rows, (int)h);
+        else
+            hipLaunchKernelGGL(rmsnorm_bwd_wide_kernel<false>, dim3((unsigned)grid), dim3(kWideThreads), 0, st, (const bf16_t*)dy, (const bf16_t*)x,
+                               (const bf16_t*)weight, (const float*)rstd, (const bf16_t*)dresidual, (bf16_t*)dx, partials, (int)rows, (int)h);
     } else {  // wider rows: two waves per row, 2 rows per block pass, two blocks per CU
         const int nchunk = ((int)h + 1023) / 1024;  // 512-column chunks per wave
         grid = (rows + 1) / 2;

@@ -380,8 +380,10 @@ def attn_bwd(q, k, v, out, dout, lse, cu_seqlens=None, scale=None):
     cu, ndocs = _cu_arg(cu_seqlens, b)
     if scale is None:
         scale = d ** -0.5
+    ws_bytes = _lib.attn_bwd_workspace_bytes(b * s, ndocs, nq, nk, d)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
     _lib.call("ezl_attn_bwd", _p(q), _p(k), _p(v), _p(out), _p(dout), _p(lse), _p(delta), _p(dq), _p(dk), _p(dv), _p(cu), ndocs,
-              b * s, s, nq, nk, d, float(scale), strides, _stream())
+              b * s, s, nq, nk, d, float(scale), strides, _p(ws), ws_bytes, _stream())
     return dq, dk, dv
 
 

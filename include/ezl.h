@@ -33,7 +33,8 @@ int ezl_version(void);
 const char* ezl_last_error(void);
 
 /* ---- RMSNorm: base_modules/layers/fused_layer_norm.py:49-71 (flash_attn rms_norm seam :56-57) ----
- * y = (x [+ residual]) * rsqrt(mean(.^2) + eps) * weight, rows of h bf16 (h % 8 == 0, h <= 8192).
+ * y = (x [+ residual]) * rsqrt(mean(.^2) + eps) * weight, rows of h bf16 (h % 8 == 0, h <= 32768; rows wider than 8192,
+ * which the reference hands to its unfused path (:56, :68-71), are read twice).
  * residual/sum_out are both NULL or both given (the residual add of llama/transformer.py:786 fused
  * in; sum_out receives x + residual rounded to bf16).  rstd: fp32 [rows], kept for backward. */
 int ezl_rmsnorm_fwd(const void* x, const void* residual, const void* weight, void* y, void* sum_out, void* rstd,
@@ -48,10 +49,10 @@ int ezl_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const voi
 /* ezl_rmsnorm_bwd without the workspace argument.  No counterpart in the reference: it exists for callers that cannot
  * obtain device memory at the call site (code under HIP graph capture, tight serving loops, harnesses that forbid
  * allocation).  The per-block dw partials go to a device array built into the library (16 MiB per GPU, held until the
- * process ends), which covers every shape ezl_rmsnorm_bwd accepts (h <= ezl_rmsnorm_bwd_noalloc_max_h() = 8192); a larger
- * h is refused with EZL_EUNSUPPORTED.  Same kernels and bit-identical results as ezl_rmsnorm_bwd.  All calls on one GPU
+ * process ends), which covers rows up to h = ezl_rmsnorm_bwd_noalloc_max_h() = 8192 (every layer width of the presets); a
+ * larger h is refused with EZL_EUNSUPPORTED.  Same kernels and bit-identical results as ezl_rmsnorm_bwd.  All calls on one GPU
  * share the array: calls that overlap on one GPU (other streams or host threads) race.  The first call on a device looks
- * the array's address up (hipGetSymbolAddress) and should therefore happen outside a graph capture. */
+ * the array's address up (hipGetSymbolAddress) and is refused with EZL_EINVAL while `stream` is recording a graph. */
 int64_t ezl_rmsnorm_bwd_noalloc_max_h(void);
 int ezl_rmsnorm_bwd_noalloc(const void* dy, const void* x, const void* weight, const void* rstd, const void* dresidual, void* dx,
                             void* dw_bf16, void* dw_f32, int accumulate, int64_t rows, int64_t h, void* stream);
@@ -126,14 +127,19 @@ int ezl_bias_grad(const void* dy, void* db_bf16, void* db_f32, int accumulate, v
  * q [T, nq, d], k/v [T, nk, d] bf16, d in {64, 128}; token n lives at
  * (n / s_len) * batch_stride + (n % s_len) * seq_stride (elements) + head * d.
  * cu_seqlens: int32 [ndocs + 1] or NULL (documents = the T / s_len batch rows; pass ndocs = T / s_len).
- * lse / delta: fp32 [nq, T].  strides (HOST pointer): fwd 8 values  q,k,v,out x (seq, batch);
- * bwd 16 values: the same 8, then dout, dq, dk, dv x (seq, batch). */
+ * lse / delta: fp32 [nq, T] (delta = rowsum(dout * out) is produced by the backward call: scratch of the caller's).
+ * strides (HOST pointer): fwd 8 values  q,k,v,out x (seq, batch); bwd 16 values: the same 8, then dout, dq, dk, dv x
+ * (seq, batch).  Backward workspace: ezl_attn_bwd_workspace_bytes() bytes, 16-byte aligned (0 for MHA: may be NULL); with
+ * a GQA group the query heads of a kv head are dealt to several workgroups whose fp32 partial dK / dV it holds, added in a
+ * fixed order (results are bit-reproducible). */
 int ezl_attn_fwd(const void* q, const void* k, const void* v, void* out, void* lse, const void* cu_seqlens, int64_t ndocs,
                  int64_t total_tokens, int64_t s_len, int64_t nq, int64_t nk, int64_t d, float scale, const int64_t* strides,
                  void* stream);
+int64_t ezl_attn_bwd_workspace_bytes(int64_t total_tokens, int64_t ndocs, int64_t nq, int64_t nk, int64_t d);
 int ezl_attn_bwd(const void* q, const void* k, const void* v, const void* out, const void* dout, const void* lse, void* delta,
                  void* dq, void* dk, void* dv, const void* cu_seqlens, int64_t ndocs, int64_t total_tokens, int64_t s_len,
-                 int64_t nq, int64_t nk, int64_t d, float scale, const int64_t* strides, void* stream);
+                 int64_t nq, int64_t nk, int64_t d, float scale, const int64_t* strides, void* workspace,
+                 int64_t workspace_bytes, void* stream);
 
 /* ---- unpadding by a key-padding mask: FlashAttention.forward, llama/transformer.py:117-141 (unpad_input / pad_input) ----
  * mask_compact: mask uint8 / bool [rows, s_len], non-zero = keep.  idx int32 [rows * s_len]: flat index of the p-th kept

@@ -46,7 +46,7 @@ def K(gpu_device):
 
 # ------------------------------------------------------------------------------------- RMSNorm
 @pytest.mark.parametrize("rows,h", [(7, 256), (1024, 688), (515, 4096), (64, 8192), (3, 8), (1537, 5120), (1030, 6144),
-                                    (2051, 8192), (5, 4104)])
+                                    (2051, 8192), (5, 4104), (300, 8200), (513, 16384), (70, 32768)])
 def test_rmsnorm_fwd_bwd(K, gpu_device, rows, h):
     print("rmsnorm", rows, h, flush=True)
     x, w, dy = rnd(rows, h, seed=1), (1 + 0.1 * torch.randn(h)).bfloat16(), rnd(rows, h, seed=2)
@@ -62,7 +62,7 @@ def test_rmsnorm_fwd_bwd(K, gpu_device, rows, h):
     close(mg, rdw + 1.0, "rmsnorm dw accumulate", rel=2e-3)
 
 
-@pytest.mark.parametrize("rows,h", [(130, 4096), (1201, 8192), (77, 5120)])
+@pytest.mark.parametrize("rows,h", [(130, 4096), (1201, 8192), (77, 5120), (259, 12288)])
 def test_add_rmsnorm_fused(K, gpu_device, rows, h):
     x, r, w = rnd(rows, h, seed=3), rnd(rows, h, seed=4), (1 + 0.1 * torch.randn(h)).bfloat16()
     y, rstd, s = K.rmsnorm_fwd(x.to(gpu_device), w.to(gpu_device), 1e-6, residual=r.to(gpu_device))
