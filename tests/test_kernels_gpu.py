@@ -197,8 +197,8 @@ def test_embedding_scatter_add_packed_batch_with_frequent_tokens(K, gpu_device):
 
 
 def test_embedding_scatter_add_with_an_id_that_fills_most_of_a_long_batch(K, gpu_device):
-    """20000 rows of which 11000 carry one id (a padding token): more than one 8192-row window of the ordering bitmap, and
-    more rows of one id than a window holds.  Row-order fp32 sums, bit for bit, in both modes."""
+    """20000 rows of which 11000 carry one id (a padding token): ten 2048-row windows of the ordering bitmap, most of them
+    more than half full, and a second id with 1500 rows.  Row-order fp32 sums, bit for bit, in both modes."""
     T, V, h = 20000, 1000, 264
     g = torch.Generator().manual_seed(6)
     ids = torch.randint(0, V, (T,), generator=g)
