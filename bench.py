@@ -195,6 +195,92 @@ def measure(name, steps, warmup, mode, input_check):
     return fig, model
 
 
+def gemm_vs_library(workload):
+    """Every GEMM launch of one training step of `workload`, this library's kernel against the box's own GEMM library
+    (torch.matmul / torch.mm -> hipBLASLt), timed alternately in one process on the same operands.  Prints a table and the
+    step's total GEMM time under three choices: this kernel everywhere, the library everywhere, the faster of the two per
+    launch -- the last is what a step could reach if every launch ran at the better of the two kernels."""
+    import torch
+    from easyllm_amd import kernels as K, workloads as W
+    w = W.WORKLOADS[workload]
+    dev = torch.device("cuda:0")
+    T, h, f, V, L = w["batch"] * w["seq"], w["hidden_size"], w["intermediate_size"], w["vocab_size"], w["num_layers"]
+    d = h // w["num_attention_heads"]
+    nq, nk = w["num_attention_heads"] * d, w["num_kv_attention_heads"] * d
+
+    def timeit(fn, n=30, warm=5):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(n):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / n * 1e3
+
+    def rnd(*shape, scale=1.0):
+        return (torch.randn(*shape, device=dev) * scale).bfloat16()
+
+    def best(a, b):  # each timed twice, alternately; the better run of each
+        ta, tb = timeit(a), timeit(b)
+        return min(ta, timeit(a)), min(tb, timeit(b))
+
+    rows = []
+
+    def fwd(name, N, Kd, count):
+        x, wt = rnd(T, Kd), rnd(N, Kd, scale=0.02)
+        rows.append((name + " forward", 2.0 * T * N * Kd, count) + best(lambda: K.linear_fwd(x, wt), lambda: torch.matmul(x, wt.t())))
+
+    def dgrad(name, outs, n_in, count):
+        dys, ws = [rnd(T, o) for o in outs], [rnd(o, n_in, scale=0.02) for o in outs]
+        dycat, wcat = torch.cat(dys, 1), torch.cat(ws, 0)
+        rows.append((name + " input gradient", 2.0 * T * n_in * sum(outs), count) +
+                    best(lambda: K.linear_dgrad_multi(dys, ws), lambda: torch.matmul(dycat, wcat)))
+
+    def wgrad(name, N, Kd, count):
+        dy, x = rnd(T, N), rnd(T, Kd)
+        mg = torch.zeros(N, Kd, device=dev, dtype=torch.float32)
+        try:
+            torch.mm(dy.t(), x, out_dtype=torch.float32)
+            lib, note = (lambda: torch.mm(dy.t(), x, out_dtype=torch.float32)), "fp32 result"
+        except Exception:
+            lib, note = (lambda: torch.matmul(dy.t(), x)), "library: bf16 result, no fp32-result call here"
+        rows.append((name + " weight gradient (%s)" % note, 2.0 * T * N * Kd, count) +
+                    best(lambda: K.linear_wgrad(dy, x, out=mg, accumulate=False), lib))
+
+    if nq == nk == h:
+        fwd("q/k/v/o", h, h, 4 * L)
+        dgrad("q+k+v (one launch)", [h, h, h], h, L)
+        dgrad("o", [h], h, L)
+        wgrad("q/k/v/o", h, h, 4 * L)
+    else:
+        fwd("q/o", nq, h, 2 * L)
+        fwd("k/v", nk, h, 2 * L)
+        dgrad("q+k+v (one launch)", [nq, nk, nk], h, L)
+        dgrad("o", [h], nq, L)
+        wgrad("q/o", nq, h, 2 * L)
+        wgrad("k/v", nk, h, 2 * L)
+    fwd("gate/up", f, h, 2 * L)
+    fwd("down", h, f, L)
+    fwd("head", V, h, 1)
+    dgrad("gate+up (one launch)", [f, f], h, L)
+    dgrad("down", [h], f, L)
+    dgrad("head", [V], h, 1)
+    wgrad("gate/up", f, h, 2 * L)
+    wgrad("down", h, f, L)
+    wgrad("head", V, h, 1)
+    print("GEMM launches of one %s step (M = %d tokens), this kernel against the library GEMM of the box" % (workload, T))
+    print("%-66s %6s %10s %11s %8s %8s" % ("launch", "count", "this us", "library us", "this TF", "lib TF"))
+    ta = tb = tm = fl = 0.0
+    for name, flops, count, a, b in rows:
+        print("%-66s %6d %10.1f %11.1f %8.0f %8.0f" % (name, count, a, b, flops / a / 1e6, flops / b / 1e6))
+        ta, tb, tm, fl = ta + count * a, tb + count * b, tm + count * min(a, b), fl + count * flops
+    for label, t in (("this kernel everywhere", ta), ("library everywhere", tb), ("faster of the two per launch", tm)):
+        print("GEMM time per step, %-30s %8.3f ms  %6.0f TFLOP/s  %.3f of the bf16 MFMA peak" % (label + ":", t / 1e3, fl / t / 1e6, fl / t / 1e6 / PEAK_BF16_TFLOPS))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -211,6 +297,8 @@ def main():
                     help="comma-separated workloads measured after the headline one (fewer steps each) and reported in the "
                          "`configs` array of the same JSON line; empty string to skip")
     ap.add_argument("--other-steps", type=int, default=6)
+    ap.add_argument("--gemm-vs-library", action="store_true",
+                    help="instead of the benchmark: time every GEMM launch of one step against the box's library GEMM and print a table")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share only (TP=1, one MI355X); --gpus %d is not supported. "
@@ -223,6 +311,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(torch.device("cuda:0"))
+    if args.gemm_vs_library:
+        gemm_vs_library(args.workload)
+        return
     fig, model = measure(args.workload, args.steps, args.warmup, args.mode, args.input_check)
     w = fig["workload"]
     out = {
