@@ -31,8 +31,8 @@ SIGNATURES = {
     "ezl_cast_f32_to_bf16": [_vp, _vp, _i64, _vp],
     "ezl_bias_add": [_vp, _vp, _vp, _i64, _i64, _vp],
     "ezl_bias_grad": [_vp, _vp, _vp, _i32, _vp, _i64, _i64, _i64, _vp],
-    "ezl_gemm_bf16": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
-    "ezl_gemm_bf16_ksplit": [_i32, _vpp, _vpp, _vp, _i64, _i64, _i64p, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
+    "ezl_gemm_bf16": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _i64, _vp],
+    "ezl_gemm_bf16_ksplit": [_i32, _vpp, _vpp, _vp, _i64, _i64, _i64p, _i64, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _i64, _vp],
     "ezl_attn_fwd": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _i64p, _vp],
     "ezl_attn_bwd": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _f32,
                      _i64p, _vp, _i64, _vp],
@@ -57,6 +57,7 @@ _SPECIAL = {
     "ezl_bias_grad_workspace_bytes": ([_i64, _i64], _i64),
     "ezl_embed_scatter_add_workspace_bytes": ([_i64, _i64], _i64),
     "ezl_attn_bwd_workspace_bytes": ([_i64, _i64, _i64, _i64, _i64], _i64),
+    "ezl_gemm_workspace_bytes": ([_i64, _i64, _i64], _i64),
     "ezl_sumsq_partials": ([], _i64),
     "ezl_location_idx_rows": ([_i64, _i64, _i64], _i64),
 }
@@ -112,6 +113,10 @@ def embed_scatter_add_workspace_bytes(rows, vocab):
 
 def attn_bwd_workspace_bytes(total_tokens, ndocs, nq, nk, d):
     return load().ezl_attn_bwd_workspace_bytes(total_tokens, ndocs, nq, nk, d)
+
+
+def gemm_workspace_bytes(M, N, K):
+    return load().ezl_gemm_workspace_bytes(M, N, K)
 
 
 def sumsq_partials():

@@ -18,6 +18,10 @@
 // phase, and the loads of tile kt+2 are issued under that phase's MFMAs.  A second kernel with register staging,
 // padded tiles and MFMA 32x32x16 covers K tails (K % 64 != 0).
 // Blocks are renumbered so that each XCD (own L2) works on a contiguous band of tiles, 8 tiles tall.
+//
+// Tile counts that leave the last round of workgroups mostly empty (320 tiles on 256 CUs, or 64 tiles in all) are evened out
+// by splitting the reduction of the tiles of that last round over several workgroups (given a workspace): each writes an
+// fp32 partial tile and a small kernel adds the partials in a fixed order, so results stay bit-reproducible.
 #include "common.h"
 
 namespace {
@@ -223,6 +227,25 @@ constexpr int DTILE = 256 * 64;  // elements per operand per stage of the swizzl
 typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(1))) const void gvoid;
 
+// tile id (in the banded order described above) -> tile coordinates
+__device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    constexpr int GROUP_M = 8;
+    const int group_size = GROUP_M * tiles_n;
+    const int group = pid / group_size;
+    const int first_m = group * GROUP_M;
+    const int gm = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
+    tm = first_m + (pid % group_size) % gm;
+    tn = (pid % group_size) / gm;
+}
+
+// Work split of a launch whose main kernel runs (K % 64 == 0): tile ids below `full` are one workgroup each; every later
+// tile is computed by `nsplit` workgroups that each take a contiguous share of the K tiles and leave an fp32 partial tile.
+struct SplitPlan {
+    int full, nsplit;
+    float* partial;  // [tiles - full][nsplit][256 x 256]
+};
+
+
 #define SG_MFMA 0x008
 #define SG_VMEM_R 0x020
 #define SG_DS_R 0x100
@@ -346,26 +369,25 @@ struct KSegments {
 template <bool A_KC, bool B_KC, typename OutT, bool MULTI = false>
 __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B, OutT* __restrict__ C,
                                                        int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
-                                                       int tiles_m, int tiles_n, const KSegments seg = KSegments()) {
+                                                       int tiles_m, int tiles_n, const SplitPlan plan, const KSegments seg = KSegments()) {
     constexpr int NW = 8, WAVES_N = 4;
     __shared__ __attribute__((aligned(1024))) bf16_t smem[4 * DTILE];  // A0 B0 A1 B1
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
-    const int nblocks = tiles_m * tiles_n;
-    int pid = blockIdx.x;
-    {
-        const int per = nblocks >> 3, rem = nblocks & 7, xcd = pid & 7, idx = pid >> 3;
+    int pid = blockIdx.x, part = 0;
+    const bool split = pid >= plan.full;
+    if (!split) {  // XCD-aware renumbering over the whole-tile workgroups
+        const int per = plan.full >> 3, rem = plan.full & 7, xcd = pid & 7, idx = pid >> 3;
         pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    } else {
+        const int u = pid - plan.full;
+        pid = plan.full + u / plan.nsplit;
+        part = u - (pid - plan.full) * plan.nsplit;
     }
-    constexpr int GROUP_M = 8;
-    const int group_size = GROUP_M * tiles_n;
-    const int group = pid / group_size;
-    const int first_m = group * GROUP_M;
-    const int gm = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
-    const int tm = first_m + (pid % group_size) % gm;
-    const int tn = (pid % group_size) / gm;
+    int tm, tn;
+    tile_of(pid, tiles_m, tiles_n, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
 
     Loader<A_KC, NW> la;
@@ -385,7 +407,11 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-    const int nk = K / BK;
+    int nk = K / BK, kt0 = 0;  // this workgroup's K tiles: kt0 .. kt0 + nk - 1
+    if (split) {
+        kt0 = (int)((int64_t)nk * part / plan.nsplit);
+        nk = (int)((int64_t)nk * (part + 1) / plan.nsplit) - kt0;
+    }
     const int64_t astep = A_KC ? BK : (int64_t)BK * lda;
     const int64_t bstep = B_KC ? BK : (int64_t)BK * ldb;
     const int arow = wm * 128, brow = wn * 64;
@@ -411,6 +437,7 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
     auto issue_tile = [&](int t, int stage) {
         const bf16_t* Ab = A;
         const bf16_t* Bb = B;
+        t += kt0;
         if constexpr (MULTI) {  // scalar selects: which pair K tile t belongs to
             const bool s1 = t >= seg.t1, s2 = t >= seg.t2;
             Ab = s2 ? seg.A2 : (s1 ? seg.A1 : A);
@@ -425,7 +452,7 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
     if (nk > 1) issue_tile(1, 1);
     // Pull the remaining kernel arguments into registers now: a scalar load still in flight inside the K loop shares the
     // counter of the LDS reads and would turn every counted wait on them into a full drain.
-    asm volatile("" ::"s"(C), "s"(ldc), "s"(accumulate));
+    asm volatile("" ::"s"(C), "s"(ldc), "s"(accumulate), "s"(plan.partial), "s"(plan.full), "s"(plan.nsplit));
     if constexpr (MULTI) asm volatile("" ::"s"(seg.A1), "s"(seg.B1), "s"(seg.A2), "s"(seg.B2), "s"(seg.t1), "s"(seg.t2));
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
     __syncthreads();
@@ -477,6 +504,15 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
 
     // epilogue: acc[i][j] register r is C[m0 + arow + 16 i + (lane & 15)][n0 + brow + 16 j + 4 (lane >> 4) + r]
     typedef typename Out4<OutT>::type out4_t;
+    if (split) {  // this workgroup's share of the reduction, as a dense fp32 tile; gemm_split_reduce_kernel adds the shares
+        float* tile = plan.partial + ((size_t)(pid - plan.full) * plan.nsplit + part) * (size_t)(BM * BN);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<f32x4*>(tile + (arow + i * 16 + (lane & 15)) * BN + brow + j * 16 + 4 * (lane >> 4)) = acc[i][j];
+        return;
+    }
     if constexpr (sizeof(OutT) == 2) {
         // bf16: 8-byte stores of 4 columns reach only half the write bandwidth of 16-byte ones (3.8 vs 6.7 TB/s on a
         // 4096 x 32000 output).  Lanes l and l ^ 16 trade halves of two neighbouring column tiles, so that the lane of
@@ -550,15 +586,91 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
 }
 
 
+
+// C tile (=|+=) sum of the nsplit fp32 partial tiles, added in index order.  One block per 16 rows of a tile: a thread owns 16
+// consecutive columns of one row.
+template <typename OutT>
+__global__ __launch_bounds__(256) void gemm_split_reduce_kernel(OutT* __restrict__ C, int M, int N, int64_t ldc, int accumulate,
+                                                                int tiles_m, int tiles_n, const SplitPlan plan) {
+    const int t = blockIdx.x >> 4;  // split tile
+    int tm, tn;
+    tile_of(plan.full + t, tiles_m, tiles_n, tm, tn);
+    const int rl = (blockIdx.x & 15) * 16 + (threadIdx.x >> 4), cl = (threadIdx.x & 15) * 16;
+    const int row = tm * BM + rl, col = tn * BN + cl;
+    if (row >= M || col >= N) return;
+    float v[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) v[e] = 0.f;
+    const float* src = plan.partial + (size_t)t * plan.nsplit * (size_t)(BM * BN) + (size_t)rl * BN + cl;
+    for (int p = 0; p < plan.nsplit; ++p, src += BM * BN) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const f32x4 x = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src) + q);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[4 * q + e] += x[e];
+        }
+    }
+    OutT* dst = C + (int64_t)row * ldc + col;
+    if (col + 16 <= N && ldc % 8 == 0 && ((uintptr_t)C & 15) == 0) {  // whole 16-column piece, 16-byte aligned
+        constexpr int VE = 16 / (int)sizeof(OutT);  // elements per 16-byte vector
+        typedef OutT vec_t __attribute__((ext_vector_type(VE)));
+#pragma unroll
+        for (int q = 0; q < 16 / VE; ++q) {
+            vec_t o;
+            if (accumulate) {
+                const vec_t old = *reinterpret_cast<const vec_t*>(dst + q * VE);
+#pragma unroll
+                for (int e = 0; e < VE; ++e) o[e] = (OutT)(v[q * VE + e] + (float)old[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < VE; ++e) o[e] = (OutT)v[q * VE + e];
+            }
+            *reinterpret_cast<vec_t*>(dst + q * VE) = o;
+        }
+        return;
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+        if (col + e < N) store_out<OutT>(dst + e, v[e], accumulate != 0);
+}
+
+// Split the tiles of a mostly empty last round?  cus workgroups run at a time (one per CU: the kernel uses 128 KiB of LDS).
+constexpr int kCus = 256;
+SplitPlan make_plan(int64_t tiles, int64_t nk, void* workspace, int64_t workspace_bytes) {
+    SplitPlan p;
+    p.full = (int)tiles; p.nsplit = 1; p.partial = nullptr;
+    const int64_t r = tiles % kCus;
+    // A last round that is more than 3/8 full is left alone: split two ways it measured slower (128 tiles, K = 4096: 88 against
+    // 81 us -- under the power limit a half-empty round runs at a higher clock, and the partial tiles cost a pass of their own).
+    if (r == 0 || r > 96) return p;
+    int s = (int)(kCus / r);
+    while (s > 1 && nk / s < 8) --s;  // a share of fewer than 8 K tiles is mostly prologue
+    if (s < 2) return p;
+    if (!workspace || workspace_bytes < r * s * (int64_t)(BM * BN) * (int64_t)sizeof(float)) return p;
+    p.full = (int)(tiles - r); p.nsplit = s; p.partial = (float*)workspace;
+    return p;
+}
+int64_t plan_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || K % BK != 0) return 0;
+    const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    SplitPlan p = make_plan(tiles, K / BK, (void*)16, INT64_MAX);
+    return p.nsplit > 1 ? (tiles - p.full) * p.nsplit * (int64_t)(BM * BN) * (int64_t)sizeof(float) : 0;
+}
+
 template <bool A_KC, bool B_KC, typename OutT>
 void launch(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
-            hipStream_t st) {
+            void* workspace, int64_t workspace_bytes, hipStream_t st) {
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const dim3 grid((unsigned)(tiles_m * tiles_n)), block(512);
-    if (K % BK == 0)
-        hipLaunchKernelGGL((gemm_d2l_kernel<A_KC, B_KC, OutT>), grid, block, 0, st, (const bf16_t*)A, (const bf16_t*)B,
-                           (OutT*)C, M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n);
-    else
+    if (K % BK == 0) {
+        const SplitPlan plan = make_plan((int64_t)tiles_m * tiles_n, K / BK, workspace, workspace_bytes);
+        const int split_tiles = tiles_m * tiles_n - plan.full;
+        hipLaunchKernelGGL((gemm_d2l_kernel<A_KC, B_KC, OutT>), dim3((unsigned)(plan.full + split_tiles * plan.nsplit)), block, 0, st,
+                           (const bf16_t*)A, (const bf16_t*)B, (OutT*)C, M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n, plan);
+        if (plan.nsplit > 1)
+            hipLaunchKernelGGL((gemm_split_reduce_kernel<OutT>), dim3((unsigned)(split_tiles * 16)), dim3(256), 0, st, (OutT*)C, M, N, ldc,
+                               accumulate, tiles_m, tiles_n, plan);
+    } else
         hipLaunchKernelGGL((gemm_staged_kernel<A_KC, B_KC, OutT, true, 2, 4>), grid, block, 0, st, (const bf16_t*)A,
                            (const bf16_t*)B, (OutT*)C, M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n);
 }
@@ -576,8 +688,12 @@ __global__ __launch_bounds__(256) void zero_c_kernel(OutT* __restrict__ C, int64
 // a_kc / b_kc: 1 if the operand's reduction index is its contiguous one
 //   A: a_kc ? A[m * lda + k] : A[k * lda + m]        B: b_kc ? B[n * ldb + k] : B[k * ldb + n]
 // out_dtype: 0 bf16, 1 fp32.  accumulate: C += A*B instead of C = A*B.
+// bytes of workspace with which a launch of this shape evens out a mostly empty last round of tiles (0: none needed)
+extern "C" int64_t ezl_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return plan_bytes(M, N, K); }
+
 extern "C" int ezl_gemm_bf16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
-                             int64_t ldc, int a_kc, int b_kc, int out_dtype, int accumulate, void* stream) {
+                             int64_t ldc, int a_kc, int b_kc, int out_dtype, int accumulate, void* workspace,
+                             int64_t workspace_bytes, void* stream) {
     EZL_REQUIRE(M >= 0 && N >= 0 && K >= 0, EZL_EINVAL, "ezl_gemm_bf16: negative size");
     EZL_REQUIRE(out_dtype == 0 || out_dtype == 1, EZL_EUNSUPPORTED, "ezl_gemm_bf16: out_dtype must be 0 (bf16) or 1 (fp32)");
     if (M == 0 || N == 0) return EZL_OK;
@@ -604,7 +720,9 @@ extern "C" int ezl_gemm_bf16(const void* A, const void* B, void* C, int64_t M, i
     const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     EZL_REQUIRE(tiles < (1LL << 31), EZL_EUNSUPPORTED, "ezl_gemm_bf16: too many tiles");
     hipStream_t st = (hipStream_t)stream;
-#define EZL_GEMM_CASE(AK, BKC, OT) launch<AK, BKC, OT>(A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, accumulate, st)
+    EZL_REQUIRE(!workspace || ezl_aligned16(workspace), EZL_EINVAL, "ezl_gemm_bf16: workspace must be 16-byte aligned");
+#define EZL_GEMM_CASE(AK, BKC, OT) \
+    launch<AK, BKC, OT>(A, B, C, (int)M, (int)N, (int)K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st)
     if (out_dtype == 0) {
         if (a_kc && b_kc) EZL_GEMM_CASE(true, true, bf16_t);
         else if (a_kc && !b_kc) EZL_GEMM_CASE(true, false, bf16_t);
@@ -627,7 +745,7 @@ extern "C" int ezl_gemm_bf16(const void* A, const void* B, void* C, int64_t M, i
 // that adds the products in fp32 and rounds once; otherwise the pairs go out as ezl_gemm_bf16 calls that accumulate into C.
 extern "C" int ezl_gemm_bf16_ksplit(int count, const void* const* A, const void* const* B, void* C, int64_t M, int64_t N,
                                     const int64_t* K, int64_t lda, int64_t ldb, int64_t ldc, int a_kc, int b_kc, int out_dtype,
-                                    int accumulate, void* stream) {
+                                    int accumulate, void* workspace, int64_t workspace_bytes, void* stream) {
     EZL_REQUIRE(count >= 1 && A && B && K, EZL_EINVAL, "ezl_gemm_bf16_ksplit: bad count or null argument array");
     bool one_launch = count <= 3 && a_kc == 1 && b_kc == 0 && out_dtype == 0 && M > 0 && N > 0;
     int64_t ktot = 0;
@@ -638,7 +756,8 @@ extern "C" int ezl_gemm_bf16_ksplit(int count, const void* const* A, const void*
     }
     if (!one_launch || count == 1) {
         for (int i = 0; i < count; ++i)
-            if (const int rc = ezl_gemm_bf16(A[i], B[i], C, M, N, K[i], lda, ldb, ldc, a_kc, b_kc, out_dtype, i == 0 ? accumulate : 1, stream))
+            if (const int rc = ezl_gemm_bf16(A[i], B[i], C, M, N, K[i], lda, ldb, ldc, a_kc, b_kc, out_dtype, i == 0 ? accumulate : 1,
+                                             workspace, workspace_bytes, stream))
                 return rc;
         return EZL_OK;
     }
@@ -660,9 +779,15 @@ extern "C" int ezl_gemm_bf16_ksplit(int count, const void* const* A, const void*
     seg.A2 = count > 2 ? (const bf16_t*)A[2] : seg.A1; seg.B2 = count > 2 ? (const bf16_t*)B[2] : seg.B1;
     seg.t2 = count > 2 ? (int)((K[0] + K[1]) / BK) : 0x7fffffff;
     const int tiles_m = (int)((M + BM - 1) / BM), tiles_n = (int)((N + BN - 1) / BN);
-    hipLaunchKernelGGL((gemm_d2l_kernel<true, false, bf16_t, true>), dim3((unsigned)tiles), dim3(512), 0, (hipStream_t)stream,
-                       (const bf16_t*)A[0], (const bf16_t*)B[0], (bf16_t*)C, (int)M, (int)N, (int)ktot, lda, ldb, ldc, accumulate, tiles_m,
-                       tiles_n, seg);
+    EZL_REQUIRE(!workspace || ezl_aligned16(workspace), EZL_EINVAL, "ezl_gemm_bf16: workspace must be 16-byte aligned");
+    const SplitPlan plan = make_plan(tiles, ktot / BK, workspace, workspace_bytes);
+    const int split_tiles = (int)tiles - plan.full;
+    hipLaunchKernelGGL((gemm_d2l_kernel<true, false, bf16_t, true>), dim3((unsigned)(plan.full + split_tiles * plan.nsplit)), dim3(512), 0,
+                       (hipStream_t)stream, (const bf16_t*)A[0], (const bf16_t*)B[0], (bf16_t*)C, (int)M, (int)N, (int)ktot, lda, ldb, ldc,
+                       accumulate, tiles_m, tiles_n, plan, seg);
+    if (plan.nsplit > 1)
+        hipLaunchKernelGGL((gemm_split_reduce_kernel<bf16_t>), dim3((unsigned)(split_tiles * 16)), dim3(256), 0, (hipStream_t)stream,
+                           (bf16_t*)C, (int)M, (int)N, ldc, accumulate, tiles_m, tiles_n, plan);
     EZL_LAUNCH_CHECK("ezl_gemm_bf16_ksplit");
     return EZL_OK;
 }

@@ -258,9 +258,16 @@ def _gemm(A, B, M, N, K, lda, ldb, a_kc, b_kc, out, out_dtype, accumulate):
         out = torch.empty(M, N, dtype=out_dtype, device=A.device)
     _need(out.is_cuda and out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (M, N), "bad GEMM output")
     _need(out.dtype in (BF16, torch.float32), "GEMM output must be bf16 or fp32")
+    ws, ws_bytes = _gemm_workspace(M, N, K, A.device)
     _lib.call("ezl_gemm_bf16", _p(A), _p(B), _p(out), M, N, K, lda, ldb, out.stride(0), 1 if a_kc else 0, 1 if b_kc else 0,
-              0 if out.dtype == BF16 else 1, 1 if accumulate else 0, _stream())
+              0 if out.dtype == BF16 else 1, 1 if accumulate else 0, _p(ws), ws_bytes, _stream())
     return out
+
+
+def _gemm_workspace(M, N, K, device):
+    """fp32 partial tiles for shapes whose last round of output tiles would leave most of the chip idle (None otherwise)."""
+    nbytes = _lib.gemm_workspace_bytes(M, N, K)
+    return (torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes) if nbytes else (None, 0)
 
 
 def linear_fwd(x2d, w):
@@ -296,9 +303,10 @@ def linear_dgrad_multi(dy2ds, ws, out=None, accumulate=False):
     if out is None:
         out = torch.empty(T, n_in, dtype=BF16, device=dy2ds[0].device)
     _need(out.is_cuda and out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (T, n_in) and out.dtype == BF16, "bad GEMM output")
+    wsp, wsp_bytes = _gemm_workspace(T, n_in, sum(w.shape[0] for w in ws), out.device)
     _lib.call("ezl_gemm_bf16_ksplit", n, (ctypes.c_void_p * n)(*[_p(dy) for dy in dy2ds]), (ctypes.c_void_p * n)(*[_p(w) for w in ws]),
               _p(out), T, n_in, (ctypes.c_int64 * n)(*[w.shape[0] for w in ws]), ldas[0], ldbs[0], out.stride(0), 1, 0, 0,
-              1 if accumulate else 0, _stream())
+              1 if accumulate else 0, _p(wsp), wsp_bytes, _stream())
     return out
 
 

@@ -105,15 +105,22 @@ int ezl_cast_f32_to_bf16(const void* in, void* out, int64_t n, void* stream);
  *      row_parallel_linear.py:113; llama/lm_head.py:62 ----
  * C[M,N] (=|+=) A * B, bf16 operands, fp32 accumulation.
  *   A: a_kc ? A[m*lda + k] : A[k*lda + m]     B: b_kc ? B[n*ldb + k] : B[k*ldb + n]
- * out_dtype 0 = bf16, 1 = fp32. */
+ * out_dtype 0 = bf16, 1 = fp32.
+ * workspace (optional, may be NULL): ezl_gemm_workspace_bytes(M, N, K) bytes of device memory, 16-byte aligned.  With it, a
+ * tile count that leaves the last round of workgroups mostly empty (320 output tiles of 256 x 256 on 256 CUs, or 64 tiles
+ * in all) is evened out: the reduction of those last tiles is split over several workgroups whose fp32 partial tiles are
+ * added in a fixed order.  Without it the same result is computed by one workgroup per tile. */
+int64_t ezl_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int ezl_gemm_bf16(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
-                  int a_kc, int b_kc, int out_dtype, int accumulate, void* stream);
+                  int a_kc, int b_kc, int out_dtype, int accumulate, void* workspace, int64_t workspace_bytes, void* stream);
 /* C (=|+=) sum_i A[i] * B[i] over `count` operand pairs with common M, N and leading dimensions and reduction lengths K[i]:
  * the input gradient sum_i dy_i W_i of the linears that share one input -- q/k/v (transformer.py:419-426) and gate/up
  * (:217-221), which the reference leaves to autograd as one matmul per linear (column_parallel_linear.py:68) plus adds.
- * One launch (fp32 sum, one rounding) for up to three pairs in the dgrad form; otherwise accumulating ezl_gemm_bf16 calls. */
+ * One launch (fp32 sum, one rounding) for up to three pairs in the dgrad form; otherwise accumulating ezl_gemm_bf16 calls.
+ * workspace as for ezl_gemm_bf16, sized by ezl_gemm_workspace_bytes(M, N, sum of K[i]). */
 int ezl_gemm_bf16_ksplit(int count, const void* const* A, const void* const* B, void* C, int64_t M, int64_t N, const int64_t* K,
-                         int64_t lda, int64_t ldb, int64_t ldc, int a_kc, int b_kc, int out_dtype, int accumulate, void* stream);
+                         int64_t lda, int64_t ldb, int64_t ldc, int a_kc, int b_kc, int out_dtype, int accumulate, void* workspace,
+                         int64_t workspace_bytes, void* stream);
 
 /* bias of a linear layer: column_parallel_linear.py:43-44 (out = x + bias) and :100 (db = sum_rows dy);
  * db goes to exactly one of db_bf16 [n] or db_f32 [n] (added to when accumulate != 0). */

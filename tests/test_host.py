@@ -32,7 +32,7 @@ def test_bad_arguments_are_rejected_without_a_gpu():
     null = ctypes.c_void_p(None)
     rc = lib.ezl_rmsnorm_fwd(null, null, null, null, null, null, 4, 12, 1e-6, null)  # h % 8 != 0
     assert rc == -2 and b"h % 8" in lib.ezl_last_error()
-    rc = lib.ezl_gemm_bf16(null, null, null, 8, 8, 8, 8, 8, 8, 1, 1, 0, 0, null)  # null operands
+    rc = lib.ezl_gemm_bf16(null, null, null, 8, 8, 8, 8, 8, 8, 1, 1, 0, 0, null, 0, null)  # null operands
     assert rc == -1
     strides = (ctypes.c_int64 * 8)(*([8] * 8))
     rc = lib.ezl_attn_fwd(null, null, null, null, null, null, 1, 16, 16, 4, 4, 96, 0.1, strides, null)  # head dim 96
