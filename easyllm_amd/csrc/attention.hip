@@ -9,8 +9,8 @@
 // contiguous inside a token, so the [s, b, heads*d] activations of the layer are consumed and
 // produced in place (no [s,b]<->[b,s] copies, cf. transformer.py:478,491).
 //
-// All three kernels use the 32x32x16 bf16 MFMA with "transposed" score tiles so that the softmax
-// statistics of a query are per-lane scalars:
+// The forward and the dK/dV kernel use the 32x32x16 bf16 MFMA, the dQ kernel the 16x16x32 one (measured faster there, slower
+// in dK/dV); all with "transposed" score tiles so that the softmax statistics of a query are per-lane scalars:
 //   forward       S^T = K Q^T (keys x queries), online softmax per lane, O^T += V^T P^T
 //   dK/dV kernel  S = Q K^T (queries x keys), dV^T += dO^T P, dK^T += Q^T dS   (block owns 128 keys)
 //   dQ kernel     S^T = K Q^T, dP^T = V dO^T, dQ^T += K^T dS^T                 (block owns 128 queries)
@@ -825,39 +825,54 @@ __global__ __launch_bounds__(kThreads) void attn_dkdv_combine_kernel(AttnParams 
 }
 
 // =================================================================================================
-// backward, dQ: a block owns 128 queries of one head and walks the keys at or before them
+// backward, dQ: a block owns 128 queries of one head (32 per wave) and walks the keys at or before them
 // =================================================================================================
+// MFMA 16x16x32: A operand lane l = row (l & 15), k = 8 (l >> 4) .. + 7; B operand lane l = column (l & 15), same k; result
+// lane l = column (l & 15), rows 4 (l >> 4) .. + 3 in four registers.  A wave owns 32 queries = two 16-query groups qg.
+//   S^T[16 keys x 16 q] = K frag (16 keys x 32 d, LDS) x Q frag (16 q x 32 d, registers), 4 d steps; likewise dP^T from V, dO
+//   dQ^T[16 d x 16 q] += K^T frag (16 d x 32 keys, transposed LDS read) x dS^T (32 keys x 16 q, from the accumulators)
+// A fragment read from LDS feeds two MFMAs (the two query groups), as one 32x32x16 fragment feeds one MFMA of twice the work.
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
 template <int D>
 __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) {
     using TL = Tile<D>;
+    constexpr int LD = TL::LD;
     __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS];  // K0 V0 K1 V1
     int doc_start, doc_len, qb;
     int bx, by;
     xcd_head_blocks(p.nq, bx, by);
-    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;  // bx = rank: longest rows first
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hq = by, hk = hq / (p.nq / p.nk);
     const int q0 = qb * 128, qw0 = q0 + wave * 32;
-    const int tok_end = doc_start + doc_len;
-    const int qi = qw0 + (lane & 31);
-    const int qtok = doc_start + (qi < doc_len ? qi : doc_len - 1);
-    bf16x8 qf[D / 16], dof[D / 16];
-    load_row_frags<D>(p.q + tok_off(qtok, p.s_len, p.q_ss, p.q_sb) + (int64_t)hq * D, lane, qf);
-    load_row_frags<D>(p.dout + tok_off(qtok, p.s_len, p.do_ss, p.do_sb) + (int64_t)hq * D, lane, dof);
-    const float lse2 = p.lse[(int64_t)hq * p.T + qtok] * kLog2e;
-    // delta = sum_d dO * O of this lane's query: the lane holds one half of the row's columns, its partner (lane ^ 32) the
-    // other.  Written out for the dK/dV kernel, which runs after this one.
-    float dlt = 0.f;
-    {
+    const int j4 = lane >> 4, l16 = lane & 15;
+    constexpr int NDS = D / 32;  // d steps of 32
+    int qi[2];
+    bf16x8 qf[2][NDS], dof[2][NDS];
+    float lse2[2], dlt[2];
+#pragma unroll
+    for (int qg = 0; qg < 2; ++qg) {
+        qi[qg] = qw0 + 16 * qg + l16;
+        const int qtok = doc_start + (qi[qg] < doc_len ? qi[qg] : doc_len - 1);
+        const bf16_t* qrow = p.q + tok_off(qtok, p.s_len, p.q_ss, p.q_sb) + (int64_t)hq * D;
+        const bf16_t* dorow = p.dout + tok_off(qtok, p.s_len, p.do_ss, p.do_sb) + (int64_t)hq * D;
         const bf16_t* orow = p.o + tok_off(qtok, p.s_len, p.o_ss, p.o_sb) + (int64_t)hq * D;
+        float acc = 0.f;
 #pragma unroll
-        for (int kd = 0; kd < D / 16; ++kd) {
-            const bf16x8 ov = *reinterpret_cast<const bf16x8*>(orow + kd * 16 + (lane >> 5) * 8);
+        for (int ds = 0; ds < NDS; ++ds) {
+            qf[qg][ds] = *reinterpret_cast<const bf16x8*>(qrow + ds * 32 + j4 * 8);
+            dof[qg][ds] = *reinterpret_cast<const bf16x8*>(dorow + ds * 32 + j4 * 8);
+            const bf16x8 ov = *reinterpret_cast<const bf16x8*>(orow + ds * 32 + j4 * 8);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) dlt += (float)ov[e] * (float)dof[kd][e];
+            for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)dof[qg][ds][e];
         }
-        dlt += __shfl_xor(dlt, 32, 64);
-        if (lane < 32 && qi < doc_len) p.delta[(int64_t)hq * p.T + doc_start + qi] = dlt;
+        // delta = sum_d dO * O of this lane's query: the four lanes l16 + 16 j hold a quarter of the row each
+        acc += __shfl_xor(acc, 16, 64);
+        acc += __shfl_xor(acc, 32, 64);
+        dlt[qg] = acc;
+        lse2[qg] = p.lse[(int64_t)hq * p.T + qtok] * kLog2e;
+        if (j4 == 0 && qi[qg] < doc_len) p.delta[(int64_t)hq * p.T + doc_start + qi[qg]] = acc;
     }
 
     const int kend = (q0 + 128 < doc_len ? q0 + 128 : doc_len);
@@ -865,7 +880,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
     const int64_t kh = (int64_t)hk * D;
     const bf16_t* kbase = p.k + tok_off(doc_start, p.s_len, p.k_ss, p.k_sb) + kh;
     const bf16_t* vbase = p.v + tok_off(doc_start, p.s_len, p.v_ss, p.v_sb) + kh;
-    // K / V tiles go from global memory straight into LDS, one tile ahead of the one being worked on
     typename TL::template Direct<kThreads / 64> kld, vld;
     kld.init(p.k_ss, lane, wave, 63);
     vld.init(p.v_ss, lane, wave, 63);
@@ -884,16 +898,33 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
         }
     };
     issue_tile(0, 0);
-    // every load issued so far (the per-lane operand rows included) has landed before the loop starts
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
 
-    f32x16 dqacc[D / 32];
+    f32x4v dqacc[D / 16][2];
 #pragma unroll
-    for (int i = 0; i < D / 32; ++i)
+    for (int i = 0; i < D / 16; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dqacc[i][r] = 0.f;
+        for (int qg = 0; qg < 2; ++qg)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dqacc[i][qg][r] = 0.f;
     const float sl2 = p.scale * kLog2e;
+
+    // A operand whose k index is d: 16 tile rows row0 .., d = 32 ds + 8 j4 .. + 7
+    auto frag_kc16 = [&](const bf16_t* s, int row0, int ds) {
+        return *reinterpret_cast<const bf16x8*>(s + (row0 + l16) * LD + ds * 32 + j4 * 8);
+    };
+    // A operand whose k index is the tile row: lane -> d column col0 + l16; k slots 8 j4 + e are tile rows krow0 + 4 j4 + e
+    // (e < 4) and krow0 + 16 + 4 j4 + e - 4 (e >= 4): the order in which two stacked 16-row accumulator tiles hold them
+    auto frag_tr16 = [&](const bf16_t* s, int krow0, int col0) {
+        const bf16_t* a = s + (krow0 + 4 * j4 + (l16 >> 2)) * LD + col0 + ((lane & 3) << 2);
+        const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(a));
+        const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(a + 16 * LD));
+        bf16x8 v;
+        v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
+        v[4] = hi[0]; v[5] = hi[1]; v[6] = hi[2]; v[7] = hi[3];
+        return v;
+    };
 
     for (int t = 0; t < ntiles; ++t) {
         const int cur = t & 1;
@@ -904,74 +935,79 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
         if (key0 <= qw0 + 31) {
             const bool on_diag = key0 + 63 > qw0;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                // S^T = K Q^T and dP^T = V dO^T in groups of 2 d-steps with the next group's fragments in flight
-                constexpr int NG = D / 32;
-                f32x16 sacc, dpacc;
-                bf16x8 fk[2][2], fvv[2][2];
-                auto ldkv = [&](int g, int buf) {
+            for (int pb = 0; pb < 2; ++pb) {  // 32 keys at a time
+                f32x4v sacc[2][2], dpacc[2][2];  // [16-key group][query group]
 #pragma unroll
-                    for (int i = 0; i < 2; ++i) {
-                        fk[buf][i] = TL::frag_kc(sK, kb * 32, g * 2 + i, lane);
-                        fvv[buf][i] = TL::frag_kc(sV, kb * 32, g * 2 + i, lane);
+                for (int kg = 0; kg < 2; ++kg)
+#pragma unroll
+                    for (int qg = 0; qg < 2; ++qg)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) { sacc[kg][qg][r] = 0.f; dpacc[kg][qg][r] = 0.f; }
+                // S^T and dP^T: per (key group, d step) one K and one V fragment, four MFMAs; next fragments in flight
+                constexpr int NST = 2 * NDS;
+                bf16x8 fk[2], fv[2];
+                auto ld = [&](int st, int buf) {
+                    fk[buf] = frag_kc16(sK, pb * 32 + (st / NDS) * 16, st % NDS);
+                    fv[buf] = frag_kc16(sV, pb * 32 + (st / NDS) * 16, st % NDS);
+                };
+                ld(0, 0);
+#pragma unroll
+                for (int st = 0; st < NST; ++st) {
+                    if (st + 1 < NST) ld(st + 1, (st + 1) & 1);
+                    const int kg = st / NDS, ds = st % NDS;
+#pragma unroll
+                    for (int qg = 0; qg < 2; ++qg) {
+                        sacc[kg][qg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fk[st & 1], qf[qg][ds], sacc[kg][qg], 0, 0, 0);
+                        dpacc[kg][qg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fv[st & 1], dof[qg][ds], dpacc[kg][qg], 0, 0, 0);
+                    }
+                }
+                // K^T fragments of the first d tiles: issued before the elementwise math
+                constexpr int NDT = D / 16;
+                bf16x8 ftk[2];
+                ftk[0] = frag_tr16(sK, pb * 32, 0);
+                bf16x8 dsf[2];
+                // register r of tile (kg, qg) <-> key key0 + 32 pb + 16 kg + 4 j4 + r, query qi[qg]; the mask is needed only on
+                // the tile that meets the diagonal (a wave-uniform property: two instantiations of the loop)
+                auto dscores = [&](auto MASKED) {
+#pragma unroll
+                    for (int qg = 0; qg < 2; ++qg) {
+#pragma unroll
+                        for (int kg = 0; kg < 2; ++kg)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kg][qg][r], sl2, -lse2[qg]));
+                                if constexpr (decltype(MASKED)::value) {
+                                    if (key0 + pb * 32 + kg * 16 + 4 * j4 + r > qi[qg]) pe = 0.f;
+                                }
+                                dsf[qg][kg * 4 + r] = (bf16_t)(pe * (dpacc[kg][qg][r] - dlt[qg]));
+                            }
                     }
                 };
-                ldkv(0, 0);
+                if (on_diag) dscores(std::true_type{});
+                else dscores(std::false_type{});
 #pragma unroll
-                for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
+                for (int dt = 0; dt < NDT; ++dt) {
+                    if (dt + 1 < NDT) ftk[(dt + 1) & 1] = frag_tr16(sK, pb * 32, (dt + 1) * 16);
 #pragma unroll
-                for (int g = 0; g < NG; ++g) {
-                    if (g + 1 < NG) ldkv(g + 1, (g + 1) & 1);
-#pragma unroll
-                    for (int i = 0; i < 2; ++i) {
-                        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fk[g & 1][i], qf[g * 2 + i], sacc, 0, 0, 0);
-                        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fvv[g & 1][i], dof[g * 2 + i], dpacc, 0, 0, 0);
-                    }
-                }
-                __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-                for (int g = 0; g < NG; ++g) {
-                    if (g + 1 < NG) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                // K^T fragments of the first 16 keys: issued before the elementwise math
-                bf16x8 ftk[2][D / 32];
-                auto ldt = [&](int tt, int buf) {
-#pragma unroll
-                    for (int db = 0; db < D / 32; ++db) ftk[buf][db] = TL::frag_tr(sK, kb * 32 + 16 * tt, db * 32, lane);
-                };
-                ldt(0, 0);
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], sl2, -lse2));
-                    if (on_diag && key0 + kb * 32 + acc_row(r, lane) > qi) pe = 0.f;
-                    dpacc[r] = pe * (dpacc[r] - dlt);
-                }
-#pragma unroll
-                for (int tt = 0; tt < 2; ++tt) {
-                    if (tt == 0) ldt(1, 1);
-                    const bf16x8 dsf = acc_to_b(dpacc, tt);
-#pragma unroll
-                    for (int db = 0; db < D / 32; ++db)
-                        dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ftk[tt][db], dsf, dqacc[db], 0, 0, 0);
+                    for (int qg = 0; qg < 2; ++qg)
+                        dqacc[dt][qg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ftk[dt & 1], dsf[qg], dqacc[dt][qg], 0, 0, 0);
                 }
             }
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of the next tile are in LDS
         __syncthreads();
     }
-    if (qi < doc_len) {
-        bf16_t* dqrow = p.dq + tok_off(doc_start + qi, p.s_len, p.dq_ss, p.dq_sb) + (int64_t)hq * D;
 #pragma unroll
-        for (int db = 0; db < D / 32; ++db)
+    for (int qg = 0; qg < 2; ++qg) {
+        if (qi[qg] >= doc_len) continue;
+        bf16_t* dqrow = p.dq + tok_off(doc_start + qi[qg], p.s_len, p.dq_ss, p.dq_sb) + (int64_t)hq * D;
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                bf16x4 w;
+        for (int dt = 0; dt < D / 16; ++dt) {
+            bf16x4 w;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) w[e] = (bf16_t)(dqacc[db][r4 * 4 + e] * p.scale);
-                *reinterpret_cast<bf16x4*>(dqrow + db * 32 + 8 * r4 + 4 * (lane >> 5)) = w;
-            }
+            for (int e = 0; e < 4; ++e) w[e] = (bf16_t)(dqacc[dt][qg][e] * p.scale);
+            *reinterpret_cast<bf16x4*>(dqrow + dt * 16 + 4 * j4) = w;
+        }
     }
 }
 
