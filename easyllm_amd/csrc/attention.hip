@@ -35,7 +35,6 @@ constexpr float kLn2 = 0.6931471805599453f;
 
 typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
 typedef __attribute__((address_space(3))) void lds_void;
-typedef __attribute__((address_space(1))) const void gvoid;
 
 struct AttnParams {
     const bf16_t* q; const bf16_t* k; const bf16_t* v; const bf16_t* o; const bf16_t* dout;
@@ -92,8 +91,13 @@ struct BlockSearch {
     }
 };
 
+// lds: kFindBlockInts ints of LDS for the search.  It is handed in by the kernel, carved from its one LDS array, instead of
+// being declared here: with several LDS variables in a kernel the compiler tags every LDS access with the variable it
+// belongs to and thereby drops the no-alias tags of the fragment reads, after which each read waits for all tile loads in
+// flight (vmcnt(0)) because it might alias their destination.
+constexpr int kFindBlockInts = 20;
 __device__ __forceinline__ bool find_block(const int* __restrict__ cu, int ndocs, int s_len, int T, int rank, int blk_rows,
-                                           int& doc_start, int& doc_len, int& blk) {
+                                           int& doc_start, int& doc_len, int& blk, int* lds) {
     const int nb_row = (s_len + blk_rows - 1) / blk_rows;
     if (!cu) {  // every piece is a whole batch row: level j holds all ndocs rows
         if (rank >= ndocs * nb_row) return false;
@@ -102,8 +106,8 @@ __device__ __forceinline__ bool find_block(const int* __restrict__ cu, int ndocs
         doc_len = s_len;
         return true;
     }
-    __shared__ int s_wave[16];
-    __shared__ int s_found[4];
+    int* s_wave = lds;        // [16]
+    int* s_found = lds + 16;  // [4]
     BlockSearch bs;
     bs.s_wave = s_wave;
     bs.tid = threadIdx.x; bs.nthr = blockDim.x; bs.lane = bs.tid & 63; bs.wv = bs.tid >> 6; bs.nwaves = bs.nthr >> 6;
@@ -216,7 +220,7 @@ struct Tile {
     static constexpr int ROWS = 64;
     static constexpr int ELEMS = ROWS * LD;
 
-    // ---- tile rows straight from global memory into LDS (global_load_lds, 16 bytes per lane) ----
+    // ---- tile rows straight from global memory into LDS (buffer_load ... lds, 16 bytes per lane) ----
     // One wave instruction fills 1 KiB of consecutive LDS, i.e. 1024 / (2 LD) padded rows: instruction q of a tile covers
     // bytes 1024 q .. 1024 q + 1023 of its LDS image, and the lane that falls on row padding re-reads the row's first chunk.
     // Rows at or past the document's end re-read its last row: finite values that only ever meet masked probabilities.
@@ -242,11 +246,14 @@ struct Tile {
         }
         // tile_rows: global address of the tile's first row (head column included); stage: its LDS image
         __device__ __forceinline__ void issue(const bf16_t* tile_rows, bf16_t* stage, int wave) const {
-            const char* g = reinterpret_cast<const char*>(tile_rows);
+            // (the buffer form of the load: while a global load to LDS is in flight the compiler, which books it as a flat
+            // access, turns every counted wait on LDS reads into a full drain)
+            const __amdgpu_buffer_rsrc_t g = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<char*>(reinterpret_cast<const char*>(tile_rows)), 0, 0xffffffffu, 0x00020000);
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
                 const int q = wave + NWAVES * j;
-                if (q < NQ) __builtin_amdgcn_global_load_lds((gvoid*)(g + off[j]), (lds_void*)(stage + q * 512), 16, 0, 0);
+                if (q < NQ) __builtin_amdgcn_raw_ptr_buffer_load_lds(g, (lds_void*)(stage + q * 512), 16, off[j], 0, 0, 0);
             }
         }
     };
@@ -262,6 +269,24 @@ struct Tile {
         const bf16_t* p = s + (krow0 + 4 * (lane >> 5) + ((lane & 15) >> 2)) * LD + col0 + (q & 1) * 16 + ((lane & 3) << 2);
         const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p));
         const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p + 8 * LD));
+        bf16x8 v;
+        v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
+        v[4] = hi[0]; v[5] = hi[1]; v[6] = hi[2]; v[7] = hi[3];
+        return v;
+    }
+    // ---- fragments of the 16x16x32 MFMA (l16 = lane & 15, j4 = lane >> 4) ----
+    // (the tile pointers are __restrict__ so that the reads carry a no-alias tag: an untagged LDS read waits for every tile
+    // load in flight)
+    // A operand whose k index is d: 16 tile rows row0 .., d = 32 ds + 8 j4 .. + 7
+    static __device__ __forceinline__ bf16x8 frag_kc16(const bf16_t* __restrict__ s, int row0, int ds, int lane) {
+        return *reinterpret_cast<const bf16x8*>(s + (row0 + (lane & 15)) * LD + ds * 32 + (lane >> 4) * 8);
+    }
+    // A operand whose k index is the tile row: lane -> d column col0 + l16; k slots 8 j4 + e are tile rows krow0 + 4 j4 + e
+    // (e < 4) and krow0 + 16 + 4 j4 + e - 4 (e >= 4): the order in which two stacked 16-row accumulator tiles hold them
+    static __device__ __forceinline__ bf16x8 frag_tr16(const bf16_t* __restrict__ s, int krow0, int col0, int lane) {
+        const bf16_t* a = s + (krow0 + 4 * (lane >> 4) + ((lane & 15) >> 2)) * LD + col0 + ((lane & 3) << 2);
+        const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(a));
+        const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(a + 16 * LD));
         bf16x8 v;
         v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
         v[4] = hi[0]; v[5] = hi[1]; v[6] = hi[2]; v[7] = hi[3];
@@ -312,11 +337,13 @@ __device__ __forceinline__ void static_for(F&& f) {
 template <int D>
 __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(AttnParams p) {
     using TL = Tile<D>;
-    __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS];  // K0 V0 K1 V1: tile t of K or V in stage t & 1
+    // K0 V0 K1 V1: tile t of K or V in stage t & 1; then the block search's scratch
+    __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS + 2 * kFindBlockInts];
     int doc_start, doc_len, qb;
     int bx, by;
     xcd_head_blocks(p.nq, bx, by);
-    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;  // bx = rank: longest rows first
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb, reinterpret_cast<int*>(smem + 4 * TL::ELEMS)))
+        return;  // bx = rank: longest rows first
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hq = by, hk = hq / (p.nq / p.nk);
     const int q0 = qb * 128, qw0 = q0 + wave * 32;
@@ -574,7 +601,8 @@ __global__ __launch_bounds__(kDkdvThreads) void attn_bwd_dkdv_kernel(AttnParams 
     int doc_start, doc_len, kbk;
     int bx, by;
     xcd_head_blocks(p.nk * p.nsplit, bx, by);
-    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, kbk)) return;
+    __shared__ int s_find[kFindBlockInts];  // (no tile loads straight into LDS in this kernel: several LDS variables do no harm)
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, kbk, s_find)) return;
     kbk = (doc_len + 127) / 128 - 1 - kbk;  // rank 0 = most blocks of queries to walk = the piece's first keys
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kg = wave & 3, half = wave >> 2;
@@ -838,11 +866,11 @@ template <int D>
 __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) {
     using TL = Tile<D>;
     constexpr int LD = TL::LD;
-    __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS];  // K0 V0 K1 V1
+    __shared__ __attribute__((aligned(16))) bf16_t smem[4 * TL::ELEMS + 2 * kFindBlockInts];  // K0 V0 K1 V1, block search scratch
     int doc_start, doc_len, qb;
     int bx, by;
     xcd_head_blocks(p.nq, bx, by);
-    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb)) return;
+    if (!find_block(p.cu, p.ndocs, p.s_len, p.T, bx, 128, doc_start, doc_len, qb, reinterpret_cast<int*>(smem + 4 * TL::ELEMS))) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hq = by, hk = hq / (p.nq / p.nk);
     const int q0 = qb * 128, qw0 = q0 + wave * 32;
@@ -910,22 +938,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
             for (int r = 0; r < 4; ++r) dqacc[i][qg][r] = 0.f;
     const float sl2 = p.scale * kLog2e;
 
-    // A operand whose k index is d: 16 tile rows row0 .., d = 32 ds + 8 j4 .. + 7
-    auto frag_kc16 = [&](const bf16_t* s, int row0, int ds) {
-        return *reinterpret_cast<const bf16x8*>(s + (row0 + l16) * LD + ds * 32 + j4 * 8);
-    };
-    // A operand whose k index is the tile row: lane -> d column col0 + l16; k slots 8 j4 + e are tile rows krow0 + 4 j4 + e
-    // (e < 4) and krow0 + 16 + 4 j4 + e - 4 (e >= 4): the order in which two stacked 16-row accumulator tiles hold them
-    auto frag_tr16 = [&](const bf16_t* s, int krow0, int col0) {
-        const bf16_t* a = s + (krow0 + 4 * j4 + (l16 >> 2)) * LD + col0 + ((lane & 3) << 2);
-        const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(a));
-        const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(a + 16 * LD));
-        bf16x8 v;
-        v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
-        v[4] = hi[0]; v[5] = hi[1]; v[6] = hi[2]; v[7] = hi[3];
-        return v;
-    };
-
     for (int t = 0; t < ntiles; ++t) {
         const int cur = t & 1;
         const bf16_t* sK = smem + cur * 2 * TL::ELEMS;
@@ -947,8 +959,8 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
                 constexpr int NST = 2 * NDS;
                 bf16x8 fk[2], fv[2];
                 auto ld = [&](int st, int buf) {
-                    fk[buf] = frag_kc16(sK, pb * 32 + (st / NDS) * 16, st % NDS);
-                    fv[buf] = frag_kc16(sV, pb * 32 + (st / NDS) * 16, st % NDS);
+                    fk[buf] = TL::frag_kc16(sK, pb * 32 + (st / NDS) * 16, st % NDS, lane);
+                    fv[buf] = TL::frag_kc16(sV, pb * 32 + (st / NDS) * 16, st % NDS, lane);
                 };
                 ld(0, 0);
 #pragma unroll
@@ -964,7 +976,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
                 // K^T fragments of the first d tiles: issued before the elementwise math
                 constexpr int NDT = D / 16;
                 bf16x8 ftk[2];
-                ftk[0] = frag_tr16(sK, pb * 32, 0);
+                ftk[0] = TL::frag_tr16(sK, pb * 32, 0, lane);
                 bf16x8 dsf[2];
                 // register r of tile (kg, qg) <-> key key0 + 32 pb + 16 kg + 4 j4 + r, query qi[qg]; the mask is needed only on
                 // the tile that meets the diagonal (a wave-uniform property: two instantiations of the loop)
@@ -987,7 +999,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
                 else dscores(std::false_type{});
 #pragma unroll
                 for (int dt = 0; dt < NDT; ++dt) {
-                    if (dt + 1 < NDT) ftk[(dt + 1) & 1] = frag_tr16(sK, pb * 32, (dt + 1) * 16);
+                    if (dt + 1 < NDT) ftk[(dt + 1) & 1] = TL::frag_tr16(sK, pb * 32, (dt + 1) * 16, lane);
 #pragma unroll
                     for (int qg = 0; qg < 2; ++qg)
                         dqacc[dt][qg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ftk[dt & 1], dsf[qg], dqacc[dt][qg], 0, 0, 0);
@@ -1010,6 +1022,15 @@ __global__ __launch_bounds__(kThreads, 2) void attn_bwd_dq_kernel(AttnParams p) 
         }
     }
 }
+// (explicit: the launches below alone have left the host-side launch stubs of some of these kernels undefined)
+template __global__ void attn_fwd_kernel<128>(AttnParams);
+template __global__ void attn_fwd_kernel<64>(AttnParams);
+template __global__ void attn_bwd_dkdv_kernel<128>(AttnParams);
+template __global__ void attn_bwd_dkdv_kernel<64>(AttnParams);
+template __global__ void attn_dkdv_combine_kernel<128>(AttnParams);
+template __global__ void attn_dkdv_combine_kernel<64>(AttnParams);
+template __global__ void attn_bwd_dq_kernel<128>(AttnParams);
+template __global__ void attn_bwd_dq_kernel<64>(AttnParams);
 
 int check_common(const char* name, int64_t T, int64_t s_len, int64_t nq, int64_t nk, int64_t d, int64_t ndocs, const int64_t* strides,
                  int nstrides) {

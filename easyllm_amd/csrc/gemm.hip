@@ -12,17 +12,20 @@
 // memory ([k][256]) and read with ds_read_b64_tr_b16 (the LDS transpose read), so nothing is ever transposed in HBM.
 //
 // Main kernel (K % 64 == 0): MFMA 16x16x32 (8x4 tiles per wave); tiles go HBM -> LDS directly
-// (global_load_lds_dwordx4, no staging registers, no ds_write); bank conflicts are avoided by an XOR swizzle applied on
+// (buffer_load_dwordx4 ... lds, no staging registers, no ds_write); bank conflicts are avoided by an XOR swizzle applied on
 // the global-address side.  A K tile is consumed in four phases (k half x M half) of 16 MFMAs; the fragments of the
 // next phase are read during the current one, the barrier that publishes the next stage sits in front of the last
 // phase, and the loads of tile kt+2 are issued under that phase's MFMAs.  A second kernel with register staging,
 // padded tiles and MFMA 32x32x16 covers K tails (K % 64 != 0).
+// The forward form on long reductions runs a 4-wave variant of the main kernel (128x128 wave tiles, one wave per SIMD).
 // Blocks are renumbered so that each XCD (own L2) works on a contiguous band of tiles, 8 tiles tall.
 //
 // Tile counts that leave the last round of workgroups mostly empty (320 tiles on 256 CUs, or 64 tiles in all) are evened out
 // by splitting the reduction of the tiles of that last round over several workgroups (given a workspace): each writes an
 // fp32 partial tile and a small kernel adds the partials in a fixed order, so results stay bit-reproducible.
 #include "common.h"
+
+#include <type_traits>
 
 namespace {
 
@@ -225,7 +228,6 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * 64) void gemm_staged_kernel(con
 constexpr int DTILE = 256 * 64;  // elements per operand per stage of the swizzled layout (32 KiB)
 
 typedef __attribute__((address_space(3))) void lds_void;
-typedef __attribute__((address_space(1))) const void gvoid;
 
 // tile id (in the banded order described above) -> tile coordinates
 __device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
@@ -250,14 +252,17 @@ struct SplitPlan {
 #define SG_VMEM_R 0x020
 #define SG_DS_R 0x100
 
-// One operand tile = 32 wave-instructions of 1 KiB each (global_load_lds_dwordx4: lane l lands at base + 16 l).
+// One operand tile = 32 wave-instructions of 1 KiB each (buffer_load_dwordx4 ... lds: lane l lands at base + 16 l).
 //   k-contiguous tile [256 rows][64 k]:  instruction q covers rows 8q..8q+7; chunk c of row r sits in slot c ^ ((r>>1)&7)
 //   k-major tile      [64 k][256 cols]:  instruction q covers k rows 2q, 2q+1; chunk c of k row sits in slot c ^ kmajor_swizzle(k)
 // Wave w issues instructions q = w*NI .. w*NI+NI-1, i.e. one contiguous NI KiB piece of the tile: M0 (the LDS base) is
 // written once per tile and the instruction offset i*1024 selects the KiB.  That offset is also added to the global
-// address, so the per-lane byte offsets are stored with i*1024 already subtracted; they are kept 4 KiB high (and the scalar
-// base 4 KiB low) so that they stay non-negative.  The address is scalar base + 32-bit lane offset + immediate: no vector
-// address arithmetic inside the K loop.
+// address, so the per-lane byte offsets are stored with i*1024 already subtracted; they are kept 4 KiB high (and the
+// buffer's base 4 KiB low) so that they stay non-negative.  The address is buffer base (scalar, advanced per K tile) +
+// 32-bit lane offset + immediate: no vector address arithmetic inside the K loop.
+// The buffer form of the load is used rather than the global one because the compiler books a global load to LDS as a
+// flat access that may touch both memories, and while one is in flight it turns every counted wait on the LDS fragment
+// reads into a full drain (lgkmcnt(0)); with buffer loads the waits inside the K loop are exact counts.
 // chunk (16 B) permutation of a k-major tile row: keeps the transpose reads of one wave instruction on distinct banks
 __device__ __forceinline__ int kmajor_swizzle(int krow) { return ((krow & 3) << 2) ^ (((krow >> 3) & 1) << 1); }
 
@@ -289,11 +294,13 @@ struct Loader {
     }
     // gbase: operand base advanced to the tile's first k, as a byte pointer
     template <int I>
-    __device__ __forceinline__ void issue_one(const char* gbase, bf16_t* piece) const {
-        __builtin_amdgcn_global_load_lds((gvoid*)(gbase - 4096 + off[I]), (lds_void*)piece, 16, I * 1024, 0);
+    __device__ __forceinline__ void issue_one(__amdgpu_buffer_rsrc_t gbase, bf16_t* piece) const {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(gbase, (lds_void*)piece, 16, off[I], 0, I * 1024, 0);
     }
     __device__ __forceinline__ void issue(const bf16_t* __restrict__ gtile, bf16_t* stage, int wave) const {
-        const char* gbase = reinterpret_cast<const char*>(gtile);
+        // an unbounded raw buffer that starts 4 KiB below the tile
+        const __amdgpu_buffer_rsrc_t gbase = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char*>(reinterpret_cast<const char*>(gtile)) - 4096, 0, 0xffffffffu, 0x00020000);
         bf16_t* piece = stage + wave * (NI * 512);
         issue_one<0>(gbase, piece);
         if constexpr (NI > 1) issue_one<1>(gbase, piece);
@@ -325,22 +332,20 @@ __device__ __forceinline__ bf16x8 sfrag(const bf16_t* __restrict__ s, int row0, 
 }
 
 // Instruction-scheduling recipe for one phase (compile-time unrolled): one MFMA, then up to PER LDS reads while reads are
-// left, then up to PER_V global->LDS loads while loads are left.
+// left, and after every LSTRIDE-th MFMA one global->LDS load while loads are left.
 template <int MASK, int N>
 __device__ __forceinline__ void sched_group() {
     if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
 }
-template <int G, int NM, int RD, int PER, int NLD, int PER_V>
+template <int G, int NM, int RD, int PER, int NLD, int LSTRIDE>
 struct SchedPhase {
     static __device__ __forceinline__ void run() {
         if constexpr (G < NM) {
             sched_group<SG_MFMA, 1>();
             constexpr int left = RD - G * PER;
-            constexpr int ds_slots = PER > 0 ? (RD + PER - 1) / PER : 0;
-            constexpr int vleft = G >= ds_slots ? NLD - (G - ds_slots) * PER_V : 0;
             sched_group<SG_DS_R, (left > PER ? PER : (left > 0 ? left : 0))>();
-            sched_group<SG_VMEM_R, (vleft > PER_V ? PER_V : (vleft > 0 ? vleft : 0))>();
-            SchedPhase<G + 1, NM, RD, PER, NLD, PER_V>::run();
+            sched_group<SG_VMEM_R, ((G % LSTRIDE == LSTRIDE - 1 && G / LSTRIDE < NLD) ? 1 : 0)>();
+            SchedPhase<G + 1, NM, RD, PER, NLD, LSTRIDE>::run();
         }
     }
 };
@@ -463,7 +468,10 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
     constexpr int NM = 16;                                // MFMAs per phase
     constexpr int NLD = 2 * (32 / NW);                    // global->LDS loads per wave and tile pair
     // phases 0 and 2 fetch the A fragments of the other M half; phases 1 and 3 fetch B and A of the next k half
-#define EZL_PHASE_SCHED(RD, LD) SchedPhase<0, NM, (RD), ((RD) + 11) / 12, (LD), 1>::run()
+#ifndef EZL_LSTRIDE
+#define EZL_LSTRIDE 2
+#endif
+#define EZL_PHASE_SCHED(RD, LD) SchedPhase<0, NM, (RD), ((RD) + 11) / 12, (LD), EZL_LSTRIDE>::run()
 #define EZL_STEP(HAS_NEXT, DO_LOAD)                                                                       \
     {                                                                                                     \
         const int cur = kt & 1;                                                                           \
@@ -586,6 +594,250 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
 }
 
 
+// =================================================================================================
+// 4-wave form of the main kernel: 2 x 2 waves, each owning 128 x 128 of the block tile
+// =================================================================================================
+// One wave per SIMD with 8 x 8 MFMA 16x16x32 tiles: the 256 accumulator registers live in AGPRs, a K tile costs a third
+// fewer LDS fragment reads than with 128 x 64 wave tiles, and nothing else runs on the SIMD to cover a stall, so the K loop
+// is laid out step by step (one MFMA per step, a sched_barrier after each):
+//   phase A of tile kt: 64 MFMAs on k half 0 (fragment set 0); the 16 fragments of k half 1 are read meanwhile
+//   wait for the loads in flight + barrier: tile kt + 1 has landed, every wave is done reading the stage of tile kt
+//   phase B of tile kt: 64 MFMAs on k half 1 (set 1); the fragments of tile kt + 1, k half 0 are read meanwhile and the
+//                       16 wave loads of tile kt + 2 go out into the stage of tile kt
+// The loop's back edge sits right behind the barrier, where no LDS read is in flight, so inside the body the compiler's
+// waits on the fragment reads are exact counts.  Reads are issued in the first half of a phase (one every second MFMA) and
+// have landed long before the next phase needs them; loads are issued one every fourth MFMA over the whole of phase B:
+// the CU's address unit takes 16 cycles per 1 KiB wave load, i.e. the four waves' loads keep it busy for all of phase B,
+// and issued any faster they fill its queue and the issuing wave stalls with its MFMAs behind it (measured on all-zero
+// operands, 4096 x 4096 x K: 0.96 us per K tile with this spacing, 1.12 with one load every second MFMA, 1.23 back to
+// back; the 8-wave kernel 1.05).  Used for the forward form (both operands k-contiguous) on whole tiles of long
+// reductions; with a k-strided operand or a short reduction the 8-wave kernel measured faster (it hides more of the
+// prologue and the epilogue).
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// one operand tile for 4 waves: wave w issues instructions q = 8 w .. 8 w + 7 (8 KiB), in two groups of four that share an
+// LDS base (the instruction offset reaches 4 KiB)
+template <bool KC>
+struct Loader4 {
+    uint32_t off[8];
+    __device__ __forceinline__ void init(int lane, int wave, int dim, int64_t ld) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int q = wave * 8 + i;
+            int64_t e;
+            if (KC) {
+                const int row = 8 * q + (lane >> 3);
+                const int c = (lane & 7) ^ ((row >> 1) & 7);
+                const int gr = row < dim ? row : dim - 1;
+                e = (int64_t)gr * ld + c * 8;
+            } else {
+                const int krow = 2 * q + (lane >> 5);
+                const int c = (lane & 31) ^ kmajor_swizzle(krow);
+                int col = c * 8;
+                col = col + 8 <= dim ? col : dim - 8;
+                e = (int64_t)krow * ld + col;
+            }
+            off[i] = (uint32_t)(e * 2 + 4096 - (i & 3) * 1024);
+        }
+    }
+    // gbase: buffer that starts 4 KiB below the tile
+    template <int I>
+    __device__ __forceinline__ void issue_one(__amdgpu_buffer_rsrc_t gbase, bf16_t* stage, int wave) const {
+        bf16_t* piece = stage + wave * 4096 + (I >> 2) * 2048;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(gbase, (lds_void*)piece, 16, off[I], 0, (I & 3) * 1024, 0);
+    }
+};
+
+// C must allow 16-byte stores (N % 8 == 0 for bf16, % 4 for fp32, ldc likewise, aligned base): the host side checks.
+template <bool A_KC, bool B_KC, typename OutT>
+__global__ __launch_bounds__(256, 1) void gemm_w4_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B, OutT* __restrict__ C,
+                                                         int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
+                                                         int tiles_m, int tiles_n) {
+    __shared__ __attribute__((aligned(1024))) bf16_t smem[4 * DTILE];  // A0 B0 A1 B1
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+
+    int pid = blockIdx.x;
+    {  // XCD-aware renumbering
+        const int nblocks = tiles_m * tiles_n;
+        const int per = nblocks >> 3, rem = nblocks & 7, xcd = pid & 7, idx = pid >> 3;
+        pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    }
+    int tm, tn;
+    tile_of(pid, tiles_m, tiles_n, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    Loader4<A_KC> la;
+    Loader4<B_KC> lb;
+    const int64_t a_blk = A_KC ? (int64_t)m0 * lda : (int64_t)m0;
+    const int64_t b_blk = B_KC ? (int64_t)n0 * ldb : (int64_t)n0;
+    la.init(lane, wave, M - m0, lda);
+    lb.init(lane, wave, N - n0, ldb);
+
+    f32x4 acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+
+    const int nk = K / BK;
+    const int64_t astep = A_KC ? BK : (int64_t)BK * lda;
+    const int64_t bstep = B_KC ? BK : (int64_t)BK * ldb;
+    const int arow = wm * 128, brow = wn * 128;
+
+    bf16x8 fa[2][8], fb[2][8];
+    // fragment f of a k half: f < 8 the B fragment f, else the A fragment f - 8
+    auto read_frag = [&](const bf16_t* sA, int ks, int buf, auto F) {
+        constexpr int f = decltype(F)::value;
+        if constexpr (f < 8) fb[buf][f] = sfrag<B_KC>(sA + DTILE, brow + f * 16, ks, lane);
+        else fa[buf][f - 8] = sfrag<A_KC>(sA, arow + (f - 8) * 16, ks, lane);
+    };
+    __amdgpu_buffer_rsrc_t ga, gb;
+    auto tile_bases = [&](int t) {
+        ga = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(reinterpret_cast<const char*>(A + a_blk + (int64_t)t * astep)) - 4096, 0,
+                                               0xffffffffu, 0x00020000);
+        gb = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(reinterpret_cast<const char*>(B + b_blk + (int64_t)t * bstep)) - 4096, 0,
+                                               0xffffffffu, 0x00020000);
+    };
+    // load l of a tile pair: l < 8 piece l of the A tile, else piece l - 8 of the B tile
+    auto issue_load = [&](int stage, auto L) {
+        constexpr int l = decltype(L)::value;
+        if constexpr (l < 8) la.template issue_one<l>(ga, smem + stage * 2 * DTILE, wave);
+        else lb.template issue_one<l - 8>(gb, smem + stage * 2 * DTILE + DTILE, wave);
+    };
+    auto issue_tile = [&](int t, int stage) {
+        tile_bases(t);
+        static_for<0, 16>([&](auto L) { issue_load(stage, L); });
+    };
+
+    issue_tile(0, 0);
+    if (nk > 1) issue_tile(1, 1);
+    // the remaining kernel arguments, pulled into registers now (a scalar load in flight inside the K loop would share the
+    // counter of the LDS reads)
+    asm volatile("" ::"s"(C), "s"(ldc), "s"(accumulate));
+    if (nk > 1) __builtin_amdgcn_s_waitcnt(0x4070);  // vmcnt(16) lgkmcnt(0): tile 0 has landed, tile 1 is still on its way
+    else __builtin_amdgcn_s_waitcnt(0x0070);         // vmcnt(0) lgkmcnt(0)
+    __syncthreads();
+    static_for<0, 16>([&](auto F) { read_frag(smem, 0, 0, F); });
+
+    constexpr int RSTEP = 2;  // a fragment read every RSTEP MFMAs (16 reads: the first half of a phase)
+    constexpr int LSTEP = 4;  // a tile load every LSTEP MFMAs (16 loads: all of phase B)
+    auto phase_a = [&](int kt) {
+        const bf16_t* sA = smem + (kt & 1) * 2 * DTILE;
+        static_for<0, 64>([&](auto S) {
+            constexpr int m = decltype(S)::value, i = m >> 3, j = m & 7;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[0][j], fa[0][i], acc[i][j], 0, 0, 0);
+            if constexpr (m % RSTEP == 0 && m / RSTEP < 16) read_frag(sA, 1, 1, std::integral_constant<int, m / RSTEP>{});
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    auto phase_b = [&](int kt, auto HAS_NEXT, auto DO_LOAD) {
+        constexpr bool has_next = decltype(HAS_NEXT)::value, do_load = decltype(DO_LOAD)::value;
+        const int cur = kt & 1;
+        const bf16_t* sN = smem + (cur ^ 1) * 2 * DTILE;
+        if constexpr (do_load) tile_bases(kt + 2);
+        static_for<0, 64>([&](auto S) {
+            constexpr int m = decltype(S)::value, i = m >> 3, j = m & 7;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[1][j], fa[1][i], acc[i][j], 0, 0, 0);
+            if constexpr (has_next && m % RSTEP == 0 && m / RSTEP < 16) read_frag(sN, 0, 0, std::integral_constant<int, m / RSTEP>{});
+            if constexpr (do_load && m % LSTEP == LSTEP - 1) issue_load(cur, std::integral_constant<int, m / LSTEP>{});
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    auto publish = [&]() {
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): the next tile has landed, this wave's reads are done
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    phase_a(0);
+    publish();
+    int kt = 0;
+    for (; kt + 2 < nk; ++kt) {
+        phase_b(kt, std::true_type{}, std::true_type{});
+        phase_a(kt + 1);
+        publish();
+    }
+    if (kt + 1 < nk) {
+        phase_b(kt, std::true_type{}, std::false_type{});
+        phase_a(kt + 1);
+        publish();
+        ++kt;
+    }
+    phase_b(kt, std::false_type{}, std::false_type{});
+
+    // the accumulators stay in their AGPRs until here (otherwise the last phase copies each finished tile out to VGPRs
+    // right behind its MFMA)
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
+
+    // epilogue: acc[i][j] register r is C[m0 + arow + 16 i + (lane & 15)][n0 + brow + 16 j + 4 (lane >> 4) + r]
+    if constexpr (sizeof(OutT) == 2) {  // lanes l and l ^ 16 trade halves of two neighbouring column tiles: 16-byte stores
+        const int g = lane >> 4;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = m0 + arow + i * 16 + (lane & 15);
+#pragma unroll
+            for (int jp = 0; jp < 4; ++jp) {
+                float lo[4], hi[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float ta = acc[i][2 * jp][r], tb = acc[i][2 * jp + 1][r];
+                    const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(ta), __float_as_uint(tb), false, false);
+                    lo[r] = __uint_as_float(sw[0]);
+                    hi[r] = __uint_as_float(sw[1]);
+                }
+                const int col = n0 + brow + (2 * jp + (g & 1)) * 16 + 8 * (g >> 1);
+                if (row >= M || col >= N) continue;
+                bf16_t* dst = C + (int64_t)row * ldc + col;
+                bf16x8 v;
+                if (accumulate) {
+                    const bf16x8 old = *reinterpret_cast<const bf16x8*>(dst);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        v[r] = (bf16_t)(lo[r] + (float)old[r]);
+                        v[4 + r] = (bf16_t)(hi[r] + (float)old[4 + r]);
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        v[r] = (bf16_t)lo[r];
+                        v[4 + r] = (bf16_t)hi[r];
+                    }
+                }
+                *reinterpret_cast<bf16x8*>(dst) = v;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = m0 + arow + i * 16 + (lane & 15);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int col = n0 + brow + j * 16 + 4 * (lane >> 4);
+                if (row >= M || col >= N) continue;
+                float* dst = C + (int64_t)row * ldc + col;
+                f32x4 v = acc[i][j];
+                if (accumulate) {
+                    const f32x4 old = *reinterpret_cast<const f32x4*>(dst);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] += old[r];
+                }
+                *reinterpret_cast<f32x4*>(dst) = v;
+            }
+        }
+    }
+}
 
 // C tile (=|+=) sum of the nsplit fp32 partial tiles, added in index order.  One block per 16 rows of a tile: a thread owns 16
 // consecutive columns of one row.
@@ -657,6 +909,10 @@ int64_t plan_bytes(int64_t M, int64_t N, int64_t K) {
     return p.nsplit > 1 ? (tiles - p.full) * p.nsplit * (int64_t)(BM * BN) * (int64_t)sizeof(float) : 0;
 }
 
+// the 4-wave kernel pays off from this many K tiles on (4096 x 4096 x K, forward form: 57 against 54 us at 32 tiles, 98
+// against 103 at 64, 179 against 194 at 128)
+constexpr int kW4MinKTiles = 48;
+
 template <bool A_KC, bool B_KC, typename OutT>
 void launch(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
             void* workspace, int64_t workspace_bytes, hipStream_t st) {
@@ -665,6 +921,14 @@ void launch(const void* A, const void* B, void* C, int M, int N, int K, int64_t 
     if (K % BK == 0) {
         const SplitPlan plan = make_plan((int64_t)tiles_m * tiles_n, K / BK, workspace, workspace_bytes);
         const int split_tiles = tiles_m * tiles_n - plan.full;
+        if constexpr (A_KC && B_KC) {
+            const int vec = 16 / (int)sizeof(OutT);
+            if (plan.nsplit <= 1 && K / BK >= kW4MinKTiles && N % vec == 0 && ldc % vec == 0 && ezl_aligned16(C)) {
+                hipLaunchKernelGGL((gemm_w4_kernel<A_KC, B_KC, OutT>), grid, dim3(256), 0, st, (const bf16_t*)A, (const bf16_t*)B, (OutT*)C,
+                                   M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n);
+                return;
+            }
+        }
         hipLaunchKernelGGL((gemm_d2l_kernel<A_KC, B_KC, OutT>), dim3((unsigned)(plan.full + split_tiles * plan.nsplit)), block, 0, st,
                            (const bf16_t*)A, (const bf16_t*)B, (OutT*)C, M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n, plan);
         if (plan.nsplit > 1)

@@ -342,6 +342,36 @@ def test_gemm_forward_with_unaligned_output_width(K, gpu_device):
         close(y, x.float() @ w.float().t(), "gemm fwd odd width")
 
 
+@pytest.mark.parametrize("T,n_in,n_out", [(512, 3072, 512), (300, 3136, 520), (1000, 4096, 264), (257, 8192, 1032)])
+def test_gemm_forward_over_long_reductions(K, gpu_device, T, n_in, n_out):
+    """The forward form (both operands k-contiguous) from 48 K tiles on runs the 4-wave kernel when the output allows 16-byte
+    stores: whole and ragged tiles, bf16 and fp32 results, overwrite and accumulate, an odd number of K tiles (3136 = 49 x 64),
+    against the fp64 product of the same bf16 operands; and bit-equal with the 8-wave kernel, which adds the K tiles in the
+    same order (reached here through an output whose row stride rules out 16-byte stores)."""
+    print("gemm long forward", T, n_in, n_out, flush=True)
+    x, w = rnd(T, n_in, seed=91), rnd(n_out, n_in, seed=92, scale=0.05)
+    xg, wg = x.to(gpu_device), w.to(gpu_device)
+    ref = (x.double() @ w.double().t())
+    y = torch.empty(T, n_out, dtype=torch.bfloat16, device=gpu_device)
+    _gemm_raw(gpu_device, xg, wg, T, n_out, n_in, 1, 1, y, False, False)
+    close(y, ref.float(), "long forward bf16")
+    base = rnd(T, n_out, seed=93)
+    y2 = base.to(gpu_device).clone()
+    _gemm_raw(gpu_device, xg, wg, T, n_out, n_in, 1, 1, y2, True, False)
+    close(y2, (ref + base.double()).float(), "long forward bf16 accumulate")
+    f = torch.full((T, n_out), 0.25, dtype=torch.float32, device=gpu_device)
+    _gemm_raw(gpu_device, xg, wg, T, n_out, n_in, 1, 1, f, True, False)
+    assert (f.double().cpu() - (ref + 0.25)).abs().max().item() <= 2e-3 * ref.abs().max().item(), "long forward fp32 accumulate"
+    _gemm_raw(gpu_device, xg, wg, T, n_out, n_in, 1, 1, f, False, False)
+    assert (f.double().cpu() - ref).abs().max().item() <= 2e-3 * ref.abs().max().item(), "long forward fp32"
+    # 8-wave kernel: a row stride of n_out + 4 elements is not a multiple of 8
+    wide = torch.zeros(T, n_out + 4, dtype=torch.bfloat16, device=gpu_device)
+    y8 = wide[:, :n_out]
+    _gemm_raw(gpu_device, xg, wg, T, n_out, n_in, 1, 1, y8, False, False)
+    assert torch.equal(y8, y), "4-wave and 8-wave kernels differ"
+    assert float(wide[:, n_out:].abs().max()) == 0.0, "wrote past the output's columns"
+
+
 def test_gemm_linearity_large(K, gpu_device):
     """Size-independent property at a full-size shape: a column block of the result equals the GEMM on that block of W --
     bit for bit where both launches sum in the same order, and to one bf16 ulp on a rare element where the narrow launch
