@@ -654,7 +654,8 @@ struct Loader4 {
     }
 };
 
-// C must allow 16-byte stores (N % 8 == 0 for bf16, % 4 for fp32, ldc likewise, aligned base): the host side checks.
+// bf16 results only; C must allow 16-byte stores (N % 8 == 0, ldc likewise, aligned base) and its tile-relative byte offsets
+// must fit 31 bits: the host side checks.
 template <bool A_KC, bool B_KC, typename OutT>
 __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B, OutT* __restrict__ C,
                                                          int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
@@ -782,61 +783,62 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(const bf16_t* __restric
         for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
 
     // epilogue: acc[i][j] register r is C[m0 + arow + 16 i + (lane & 15)][n0 + brow + 16 j + 4 (lane >> 4) + r]
-    if constexpr (sizeof(OutT) == 2) {  // lanes l and l ^ 16 trade halves of two neighbouring column tiles: 16-byte stores
-        const int g = lane >> 4;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int row = m0 + arow + i * 16 + (lane & 15);
+    // C is addressed as a buffer that starts at the tile's corner and ends behind the tile's last valid row: a store to a row
+    // past M drops out by the buffer's range check, one to a column past N by an offset that is out of range.  The epilogue is
+    // thus straight-line code (no branch per store, and `accumulate` decided once), whose 32 independent chains of
+    // register moves, conversions and stores the compiler interleaves; with a branch per store it took twice as long.
+    static_assert(sizeof(OutT) == 2, "bf16 results");
+    constexpr int SZ = 2;
+    const int mrem = M - m0 < BM ? M - m0 : BM;
+    const __amdgpu_buffer_rsrc_t cbuf = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<char*>(C + (int64_t)m0 * ldc + n0), 0, (uint32_t)(((int64_t)mrem * ldc - n0) * SZ), 0x00020000);
+    const uint32_t row_off = (uint32_t)(arow + (lane & 15)) * (uint32_t)(ldc * SZ);
+    const uint32_t row_step = (uint32_t)(16 * ldc * SZ);  // scalar: rows 16 i
+    constexpr uint32_t kOut = 0x80000000u;
+    auto epilogue = [&](auto ACC) {
+        constexpr bool accum = decltype(ACC)::value;
+        {  // lanes l and l ^ 16 trade halves of two neighbouring column tiles: 16-byte stores
+            const int g = lane >> 4;
+            uint32_t voff[4];
 #pragma unroll
             for (int jp = 0; jp < 4; ++jp) {
-                float lo[4], hi[4];
+                const int col = brow + (2 * jp + (g & 1)) * 16 + 8 * (g >> 1);
+                voff[jp] = n0 + col < N ? row_off + (uint32_t)col * SZ : kOut;
+            }
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float ta = acc[i][2 * jp][r], tb = acc[i][2 * jp + 1][r];
-                    const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(ta), __float_as_uint(tb), false, false);
-                    lo[r] = __uint_as_float(sw[0]);
-                    hi[r] = __uint_as_float(sw[1]);
-                }
-                const int col = n0 + brow + (2 * jp + (g & 1)) * 16 + 8 * (g >> 1);
-                if (row >= M || col >= N) continue;
-                bf16_t* dst = C + (int64_t)row * ldc + col;
-                bf16x8 v;
-                if (accumulate) {
-                    const bf16x8 old = *reinterpret_cast<const bf16x8*>(dst);
+            for (int i = 0; i < 8; ++i) {
+#pragma unroll
+                for (int jp = 0; jp < 4; ++jp) {
+                    float lo[4], hi[4];
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        v[r] = (bf16_t)(lo[r] + (float)old[r]);
-                        v[4 + r] = (bf16_t)(hi[r] + (float)old[4 + r]);
+                        const float ta = acc[i][2 * jp][r], tb = acc[i][2 * jp + 1][r];
+                        const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(ta), __float_as_uint(tb), false, false);
+                        lo[r] = __uint_as_float(sw[0]);
+                        hi[r] = __uint_as_float(sw[1]);
                     }
-                } else {
+                    bf16x8 v;
+                    if constexpr (accum) {
+                        const bf16x8 old = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(cbuf, voff[jp], i * row_step, 0));
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        v[r] = (bf16_t)lo[r];
-                        v[4 + r] = (bf16_t)hi[r];
+                        for (int r = 0; r < 4; ++r) {
+                            v[r] = (bf16_t)(lo[r] + (float)old[r]);
+                            v[4 + r] = (bf16_t)(hi[r] + (float)old[4 + r]);
+                        }
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            v[r] = (bf16_t)lo[r];
+                            v[4 + r] = (bf16_t)hi[r];
+                        }
                     }
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), cbuf, voff[jp], i * row_step, 0);
                 }
-                *reinterpret_cast<bf16x8*>(dst) = v;
             }
         }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int row = m0 + arow + i * 16 + (lane & 15);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int col = n0 + brow + j * 16 + 4 * (lane >> 4);
-                if (row >= M || col >= N) continue;
-                float* dst = C + (int64_t)row * ldc + col;
-                f32x4 v = acc[i][j];
-                if (accumulate) {
-                    const f32x4 old = *reinterpret_cast<const f32x4*>(dst);
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) v[r] += old[r];
-                }
-                *reinterpret_cast<f32x4*>(dst) = v;
-            }
-        }
-    }
+    };
+    if (accumulate) epilogue(std::true_type{});
+    else epilogue(std::false_type{});
 }
 
 // C tile (=|+=) sum of the nsplit fp32 partial tiles, added in index order.  One block per 16 rows of a tile: a thread owns 16
@@ -921,9 +923,10 @@ void launch(const void* A, const void* B, void* C, int M, int N, int K, int64_t 
     if (K % BK == 0) {
         const SplitPlan plan = make_plan((int64_t)tiles_m * tiles_n, K / BK, workspace, workspace_bytes);
         const int split_tiles = tiles_m * tiles_n - plan.full;
-        if constexpr (A_KC && B_KC) {
-            const int vec = 16 / (int)sizeof(OutT);
-            if (plan.nsplit <= 1 && K / BK >= kW4MinKTiles && N % vec == 0 && ldc % vec == 0 && ezl_aligned16(C)) {
+        if constexpr (A_KC && B_KC && sizeof(OutT) == 2) {
+            const int vec = 8;
+            if (plan.nsplit <= 1 && K / BK >= kW4MinKTiles && N % vec == 0 && ldc % vec == 0 && ezl_aligned16(C) &&
+                (int64_t)ldc * (int64_t)sizeof(OutT) * BM < (1LL << 31)) {  // tile-relative byte offsets of C fit 31 bits
                 hipLaunchKernelGGL((gemm_w4_kernel<A_KC, B_KC, OutT>), grid, dim3(256), 0, st, (const bf16_t*)A, (const bf16_t*)B, (OutT*)C,
                                    M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n);
                 return;
