@@ -659,17 +659,21 @@ struct Loader4 {
 template <bool A_KC, bool B_KC, typename OutT>
 __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B, OutT* __restrict__ C,
                                                          int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
-                                                         int tiles_m, int tiles_n) {
+                                                         int tiles_m, int tiles_n, const SplitPlan plan) {
     __shared__ __attribute__((aligned(1024))) bf16_t smem[4 * DTILE];  // A0 B0 A1 B1
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
 
-    int pid = blockIdx.x;
-    {  // XCD-aware renumbering
-        const int nblocks = tiles_m * tiles_n;
-        const int per = nblocks >> 3, rem = nblocks & 7, xcd = pid & 7, idx = pid >> 3;
+    int pid = blockIdx.x, part = 0;
+    const bool split = pid >= plan.full;
+    if (!split) {  // XCD-aware renumbering over the whole-tile workgroups
+        const int per = plan.full >> 3, rem = plan.full & 7, xcd = pid & 7, idx = pid >> 3;
         pid = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    } else {  // a tile of the split last round: this workgroup's share of its K tiles
+        const int u = pid - plan.full;
+        pid = plan.full + u / plan.nsplit;
+        part = u - (pid - plan.full) * plan.nsplit;
     }
     int tm, tn;
     tile_of(pid, tiles_m, tiles_n, tm, tn);
@@ -690,7 +694,11 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(const bf16_t* __restric
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-    const int nk = K / BK;
+    int nk = K / BK, kt0 = 0;  // this workgroup's K tiles: kt0 .. kt0 + nk - 1
+    if (split) {
+        kt0 = (int)((int64_t)nk * part / plan.nsplit);
+        nk = (int)((int64_t)nk * (part + 1) / plan.nsplit) - kt0;
+    }
     const int64_t astep = A_KC ? BK : (int64_t)BK * lda;
     const int64_t bstep = B_KC ? BK : (int64_t)BK * ldb;
     const int arow = wm * 128, brow = wn * 128;
@@ -704,6 +712,7 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(const bf16_t* __restric
     };
     __amdgpu_buffer_rsrc_t ga, gb;
     auto tile_bases = [&](int t) {
+        t += kt0;
         ga = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(reinterpret_cast<const char*>(A + a_blk + (int64_t)t * astep)) - 4096, 0,
                                                0xffffffffu, 0x00020000);
         gb = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(reinterpret_cast<const char*>(B + b_blk + (int64_t)t * bstep)) - 4096, 0,
@@ -724,7 +733,7 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(const bf16_t* __restric
     if (nk > 1) issue_tile(1, 1);
     // the remaining kernel arguments, pulled into registers now (a scalar load in flight inside the K loop would share the
     // counter of the LDS reads)
-    asm volatile("" ::"s"(C), "s"(ldc), "s"(accumulate));
+    asm volatile("" ::"s"(C), "s"(ldc), "s"(accumulate), "s"(plan.partial), "s"(plan.full), "s"(plan.nsplit));
     if (nk > 1) __builtin_amdgcn_s_waitcnt(0x4070);  // vmcnt(16) lgkmcnt(0): tile 0 has landed, tile 1 is still on its way
     else __builtin_amdgcn_s_waitcnt(0x0070);         // vmcnt(0) lgkmcnt(0)
     __syncthreads();
@@ -775,6 +784,15 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(const bf16_t* __restric
     }
     phase_b(kt, std::false_type{}, std::false_type{});
 
+    if (split) {  // this workgroup's share of the reduction, as a dense fp32 tile; gemm_split_reduce_kernel adds the shares
+        float* tile = plan.partial + ((size_t)(pid - plan.full) * plan.nsplit + part) * (size_t)(BM * BN);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                *reinterpret_cast<f32x4*>(tile + (arow + i * 16 + (lane & 15)) * BN + brow + j * 16 + 4 * (lane >> 4)) = acc[i][j];
+        return;
+    }
     // the accumulators stay in their AGPRs until here (otherwise the last phase copies each finished tile out to VGPRs
     // right behind its MFMA)
 #pragma unroll
@@ -925,10 +943,15 @@ void launch(const void* A, const void* B, void* C, int M, int N, int K, int64_t 
         const int split_tiles = tiles_m * tiles_n - plan.full;
         if constexpr (A_KC && B_KC && sizeof(OutT) == 2) {
             const int vec = 8;
-            if (plan.nsplit <= 1 && K / BK >= kW4MinKTiles && N % vec == 0 && ldc % vec == 0 && ezl_aligned16(C) &&
+            // (a launch that is split tiles only is judged by the length of a share)
+            const int w4_ktiles = plan.nsplit > 1 && plan.full == 0 ? K / BK / plan.nsplit : K / BK;
+            if (w4_ktiles >= kW4MinKTiles && N % vec == 0 && ldc % vec == 0 && ezl_aligned16(C) &&
                 (int64_t)ldc * (int64_t)sizeof(OutT) * BM < (1LL << 31)) {  // tile-relative byte offsets of C fit 31 bits
-                hipLaunchKernelGGL((gemm_w4_kernel<A_KC, B_KC, OutT>), grid, dim3(256), 0, st, (const bf16_t*)A, (const bf16_t*)B, (OutT*)C,
-                                   M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n);
+                hipLaunchKernelGGL((gemm_w4_kernel<A_KC, B_KC, OutT>), dim3((unsigned)(plan.full + split_tiles * plan.nsplit)), dim3(256), 0, st,
+                                   (const bf16_t*)A, (const bf16_t*)B, (OutT*)C, M, N, K, lda, ldb, ldc, accumulate, tiles_m, tiles_n, plan);
+                if (plan.nsplit > 1)
+                    hipLaunchKernelGGL((gemm_split_reduce_kernel<OutT>), dim3((unsigned)(split_tiles * 16)), dim3(256), 0, st, (OutT*)C, M, N,
+                                       ldc, accumulate, tiles_m, tiles_n, plan);
                 return;
             }
         }

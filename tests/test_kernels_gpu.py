@@ -279,7 +279,7 @@ def _gemm_raw(gpu_device, A, B, M, N, Kd, a_kc, b_kc, out, accumulate, with_work
     return nbytes
 
 
-@pytest.mark.parametrize("T,n_in,n_out", [(4096, 2048, 5120), (1000, 4096, 520), (4096, 8192, 1024)])
+@pytest.mark.parametrize("T,n_in,n_out", [(4096, 2048, 5120), (1000, 4096, 520), (4096, 8192, 1024), (4096, 3072, 5120)])
 def test_gemm_with_a_split_last_round_of_tiles(K, gpu_device, T, n_in, n_out):
     """Tile counts that leave the last round of 256 workgroups mostly empty (320 tiles; 12 tiles with ragged edges; 64 tiles):
     with the workspace the reduction of those tiles is split over several workgroups.  All three operand forms against the
