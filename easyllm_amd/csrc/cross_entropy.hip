@@ -289,22 +289,28 @@ __global__ __launch_bounds__(kCeBlock) void ce_fused_reg_kernel(const bf16_t* __
 // once.  The first 9 x 1024 vectors of 8 logits live in LDS (144 KiB, thread t owns vector t of every 1024: private
 // slots, no barriers), the remaining NR x 1024 in registers.  exp is evaluated twice per element (sum pass, gradient
 // pass): fp32 copies would not fit.  While the gradient pass runs, each finished vector's slot is refilled with the
-// block's next row -- registers by a plain load, LDS slots by global_load_lds, which needs no registers at all -- so the
-// HBM pipe is busy under the vector ALU work.  Vectors past the row end hold -inf (exp = 0) and are never stored.
+// block's next row -- registers by a plain load, LDS slots by a buffer load straight to LDS, which needs no registers at
+// all -- so the HBM pipe is busy under the vector ALU work.  Vectors past the row end hold -inf (exp = 0) and are never
+// stored.  For the refills to stay in flight while later slots are read, the LDS reads must not wait for them: the kernel
+// has a single LDS array (the reduction cells sit behind the row) and reads it through a __restrict__ pointer, which keeps
+// the reads' no-alias tag (with a second LDS variable the compiler re-tags every access and each read then waits for all
+// loads in flight, vmcnt(0)); and the loads are buffer loads, because a global load to LDS in flight turns every counted
+// wait on LDS reads into a full drain.
 constexpr int kWideBlock = 1024;
 constexpr int kWideWaves = kWideBlock / 64;
 constexpr int kWideLds = 9;  // vectors per thread kept in LDS
 
 typedef __attribute__((address_space(3))) void ce_lds_void;
-typedef __attribute__((address_space(1))) const void ce_gvoid;
+
+__device__ __forceinline__ bf16x8 ce_lds_vec(const bf16_t* __restrict__ row, int i) { return *reinterpret_cast<const bf16x8*>(row + i * 8); }
 
 template <int NR, bool HAS_CUT>
 __global__ __launch_bounds__(kWideBlock) void ce_fused_wide_kernel(const bf16_t* __restrict__ logits, const int64_t* __restrict__ labels,
                                                                    const float* __restrict__ weights, const float* __restrict__ count,
                                                                    float* __restrict__ loss, bf16_t* __restrict__ grad, int64_t rows,
                                                                    int V, int vend) {
-    __shared__ __attribute__((aligned(16))) bf16_t srow[kWideLds * kWideBlock * 8];
-    __shared__ float red[2][kWideWaves];
+    __shared__ __attribute__((aligned(16))) bf16_t srow[kWideLds * kWideBlock * 8 + 4 * kWideWaves];  // the row, then red[2][waves]
+    float* red = reinterpret_cast<float*>(srow + kWideLds * kWideBlock * 8);
     const int v8 = V >> 3;  // >= kWideLds * kWideBlock (checked by the host): every LDS vector lies inside the row
     const float inv_n = 1.0f / count[0];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -320,10 +326,11 @@ __global__ __launch_bounds__(kWideBlock) void ce_fused_wide_kernel(const bf16_t*
         }
     };
     auto fetch_lds = [&](const bf16_t* src, int j) {  // one wave instruction fills the 64 slots of this wave in chunk j
-        __builtin_amdgcn_global_load_lds((ce_gvoid*)(src + (int64_t)(tid + j * kWideBlock) * 8),
-                                         (ce_lds_void*)(srow + (j * kWideBlock + wv * 64) * 8), 16, 0, 0);
+        const __amdgpu_buffer_rsrc_t g = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(src), 0, 0xffffffffu, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(g, (ce_lds_void*)(srow + (j * kWideBlock + wv * 64) * 8), 16, tid * 16,
+                                                 j * kWideBlock * 16, 0, 0);
     };
-    auto lds_vec = [&](int j) { return *reinterpret_cast<const bf16x8*>(srow + (tid + j * kWideBlock) * 8); };
+    auto lds_vec = [&](int j) { return ce_lds_vec(srow, tid + j * kWideBlock); };
 
     int64_t r = blockIdx.x;
     if (r < rows) {
@@ -378,11 +385,11 @@ __global__ __launch_bounds__(kWideBlock) void ce_fused_wide_kernel(const bf16_t*
         for (int j = 0; j < NR; ++j) max_of(raw[j], tid + (kWideLds + j) * kWideBlock);
         m = wave_max(m);
         __syncthreads();  // red is free again (read by every thread at the end of the previous row)
-        if (lane == 0) red[0][wv] = m;
+        if (lane == 0) red[wv] = m;
         __syncthreads();
-        m = red[0][0];
+        m = red[0];
 #pragma unroll
-        for (int i = 1; i < kWideWaves; ++i) m = fmaxf(m, red[0][i]);
+        for (int i = 1; i < kWideWaves; ++i) m = fmaxf(m, red[i]);
         const float mb = m * kLog2e;
         // ---- pass 2: sum of exp(x - max) over the columns below vend
         float ssum = 0.f;
@@ -403,11 +410,11 @@ __global__ __launch_bounds__(kWideBlock) void ce_fused_wide_kernel(const bf16_t*
             sum_of(raw[j], tid + (kWideLds + j) * kWideBlock);
         }
         ssum = wave_sum(ssum);
-        if (lane == 0) red[1][wv] = ssum;
+        if (lane == 0) red[kWideWaves + wv] = ssum;
         __syncthreads();
         ssum = 0.f;
 #pragma unroll
-        for (int i = 0; i < kWideWaves; ++i) ssum += red[1][i];
+        for (int i = 0; i < kWideWaves; ++i) ssum += red[kWideWaves + i];
         const float lse = m + logf(ssum);
         if (tid == 0) loss[r] = masked ? logf(ssum) : (lse - xt);
         const float scale = w * inv_n;
