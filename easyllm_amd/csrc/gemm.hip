@@ -332,20 +332,22 @@ __device__ __forceinline__ bf16x8 sfrag(const bf16_t* __restrict__ s, int row0, 
 }
 
 // Instruction-scheduling recipe for one phase (compile-time unrolled): one MFMA, then up to PER LDS reads while reads are
-// left, and after every LSTRIDE-th MFMA one global->LDS load while loads are left.
+// left, then up to PER_V global->LDS loads while loads are left.
 template <int MASK, int N>
 __device__ __forceinline__ void sched_group() {
     if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
 }
-template <int G, int NM, int RD, int PER, int NLD, int LSTRIDE>
+template <int G, int NM, int RD, int PER, int NLD, int PER_V>
 struct SchedPhase {
     static __device__ __forceinline__ void run() {
         if constexpr (G < NM) {
             sched_group<SG_MFMA, 1>();
             constexpr int left = RD - G * PER;
+            constexpr int ds_slots = PER > 0 ? (RD + PER - 1) / PER : 0;
+            constexpr int vleft = G >= ds_slots ? NLD - (G - ds_slots) * PER_V : 0;
             sched_group<SG_DS_R, (left > PER ? PER : (left > 0 ? left : 0))>();
-            sched_group<SG_VMEM_R, ((G % LSTRIDE == LSTRIDE - 1 && G / LSTRIDE < NLD) ? 1 : 0)>();
-            SchedPhase<G + 1, NM, RD, PER, NLD, LSTRIDE>::run();
+            sched_group<SG_VMEM_R, (vleft > PER_V ? PER_V : (vleft > 0 ? vleft : 0))>();
+            SchedPhase<G + 1, NM, RD, PER, NLD, PER_V>::run();
         }
     }
 };
@@ -468,10 +470,7 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
     constexpr int NM = 16;                                // MFMAs per phase
     constexpr int NLD = 2 * (32 / NW);                    // global->LDS loads per wave and tile pair
     // phases 0 and 2 fetch the A fragments of the other M half; phases 1 and 3 fetch B and A of the next k half
-#ifndef EZL_LSTRIDE
-#define EZL_LSTRIDE 2
-#endif
-#define EZL_PHASE_SCHED(RD, LD) SchedPhase<0, NM, (RD), ((RD) + 11) / 12, (LD), EZL_LSTRIDE>::run()
+#define EZL_PHASE_SCHED(RD, LD) SchedPhase<0, NM, (RD), ((RD) + 11) / 12, (LD), 1>::run()
 #define EZL_STEP(HAS_NEXT, DO_LOAD)                                                                       \
     {                                                                                                     \
         const int cur = kt & 1;                                                                           \
