@@ -17,7 +17,8 @@
 // next phase are read during the current one, the barrier that publishes the next stage sits in front of the last
 // phase, and the loads of tile kt+2 are issued under that phase's MFMAs.  A second kernel with register staging,
 // padded tiles and MFMA 32x32x16 covers K tails (K % 64 != 0).
-// The forward form on long reductions runs a 4-wave variant of the main kernel (128x128 wave tiles, one wave per SIMD).
+// The forward form and the fp32 weight-gradient form on long reductions run a 4-wave variant of the main kernel (128x128
+// wave tiles, one wave per SIMD).
 // Blocks are renumbered so that each XCD (own L2) works on a contiguous band of tiles, 8 tiles tall.
 //
 // Tile counts that leave the last round of workgroups mostly empty (320 tiles on 256 CUs, or 64 tiles in all) are evened out
@@ -609,9 +610,9 @@ __global__ __launch_bounds__(512) void gemm_d2l_kernel(const bf16_t* __restrict_
 // the CU's address unit takes 16 cycles per 1 KiB wave load, i.e. the four waves' loads keep it busy for all of phase B,
 // and issued any faster they fill its queue and the issuing wave stalls with its MFMAs behind it (measured on all-zero
 // operands, 4096 x 4096 x K: 0.96 us per K tile with this spacing, 1.12 with one load every second MFMA, 1.23 back to
-// back; the 8-wave kernel 1.05).  Used for the forward form (both operands k-contiguous) on whole tiles of long
-// reductions; with a k-strided operand or a short reduction the 8-wave kernel measured faster (it hides more of the
-// prologue and the epilogue).
+// back; the 8-wave kernel 1.05).  Used for the forward form (both operands k-contiguous, bf16 result) and for the
+// weight-gradient form with an fp32 result on long reductions; for input gradients and short reductions the 8-wave
+// kernel, which hides more of the prologue and the epilogue, is as fast or faster.
 template <int I, int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
     if constexpr (I < N) {
@@ -653,8 +654,8 @@ struct Loader4 {
     }
 };
 
-// bf16 results only; C must allow 16-byte stores (N % 8 == 0, ldc likewise, aligned base) and its tile-relative byte offsets
-// must fit 31 bits: the host side checks.
+// C must allow 16-byte stores (N and ldc multiples of 8 for bf16, of 4 for fp32, aligned base) and, for bf16, its
+// tile-relative byte offsets must fit 31 bits: the host side checks.
 template <bool A_KC, bool B_KC, typename OutT>
 __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ B, OutT* __restrict__ C,
                                                          int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc, int accumulate,
@@ -793,18 +794,36 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(const bf16_t* __restric
         return;
     }
     // the accumulators stay in their AGPRs until here (otherwise the last phase copies each finished tile out to VGPRs
-    // right behind its MFMA)
+    // right behind its MFMA and runs out of registers)
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
+    if constexpr (sizeof(OutT) == 4) {  // fp32 results (weight gradients): the 4 columns a lane owns as one 16-byte store
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = m0 + arow + i * 16 + (lane & 15);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int col = n0 + brow + j * 16 + 4 * (lane >> 4);
+                if (row >= M || col >= N) continue;
+                float* dst = C + (int64_t)row * ldc + col;
+                f32x4 v = acc[i][j];
+                if (accumulate) {
+                    const f32x4 old = *reinterpret_cast<const f32x4*>(dst);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] += old[r];
+                }
+                *reinterpret_cast<f32x4*>(dst) = v;
+            }
+        }
+    } else {
 
     // epilogue: acc[i][j] register r is C[m0 + arow + 16 i + (lane & 15)][n0 + brow + 16 j + 4 (lane >> 4) + r]
     // C is addressed as a buffer that starts at the tile's corner and ends behind the tile's last valid row: a store to a row
     // past M drops out by the buffer's range check, one to a column past N by an offset that is out of range.  The epilogue is
     // thus straight-line code (no branch per store, and `accumulate` decided once), whose 32 independent chains of
     // register moves, conversions and stores the compiler interleaves; with a branch per store it took twice as long.
-    static_assert(sizeof(OutT) == 2, "bf16 results");
     constexpr int SZ = 2;
     const int mrem = M - m0 < BM ? M - m0 : BM;
     const __amdgpu_buffer_rsrc_t cbuf = __builtin_amdgcn_make_buffer_rsrc(
@@ -856,6 +875,7 @@ __global__ __launch_bounds__(256, 1) void gemm_w4_kernel(const bf16_t* __restric
     };
     if (accumulate) epilogue(std::true_type{});
     else epilogue(std::false_type{});
+    }
 }
 
 // C tile (=|+=) sum of the nsplit fp32 partial tiles, added in index order.  One block per 16 rows of a tile: a thread owns 16
@@ -940,8 +960,11 @@ void launch(const void* A, const void* B, void* C, int M, int N, int K, int64_t 
     if (K % BK == 0) {
         const SplitPlan plan = make_plan((int64_t)tiles_m * tiles_n, K / BK, workspace, workspace_bytes);
         const int split_tiles = tiles_m * tiles_n - plan.full;
-        if constexpr (A_KC && B_KC && sizeof(OutT) == 2) {
-            const int vec = 8;
+        // The 4-wave kernel: forward form with a bf16 result, and weight-gradient form with an fp32 result (inside the steps
+        // 0.4 - 0.8 % faster than the 8-wave kernel although a single launch at K = 4096 is not: it moves a third fewer LDS
+        // bytes, and the steps are bound by power).  With a k-strided B only (input gradients) it gained nothing.
+        if constexpr ((A_KC && B_KC && sizeof(OutT) == 2) || (!A_KC && !B_KC && sizeof(OutT) == 4)) {
+            const int vec = 16 / (int)sizeof(OutT);
             // (a launch that is split tiles only is judged by the length of a share)
             const int w4_ktiles = plan.nsplit > 1 && plan.full == 0 ? K / BK / plan.nsplit : K / BK;
             if (w4_ktiles >= kW4MinKTiles && N % vec == 0 && ldc % vec == 0 && ezl_aligned16(C) &&

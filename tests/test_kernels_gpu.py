@@ -372,6 +372,28 @@ def test_gemm_forward_over_long_reductions(K, gpu_device, T, n_in, n_out):
     assert float(wide[:, n_out:].abs().max()) == 0.0, "wrote past the output's columns"
 
 
+@pytest.mark.parametrize("T,n_in,n_out", [(3072, 512, 512), (3136, 520, 264), (8192, 264, 1032)])
+def test_gemm_fp32_weight_gradient_over_many_tokens(K, gpu_device, T, n_in, n_out):
+    """The fp32 weight gradient (both operands k-strided) over 48 K tiles or more runs the 4-wave kernel: whole and ragged
+    tiles, an odd number of K tiles, overwrite and accumulate, against the fp64 product of the same bf16 operands; and
+    bit-equal with the 8-wave kernel (same order of the K tiles), reached through a row stride that rules out 16-byte stores."""
+    print("gemm long wgrad", T, n_in, n_out, flush=True)
+    x, dy = rnd(T, n_in, seed=95), rnd(T, n_out, seed=96)
+    xg, dyg = x.to(gpu_device), dy.to(gpu_device)
+    ref = dy.double().t() @ x.double()
+    tol = 2e-3 * ref.abs().max().item()
+    g = torch.full((n_out, n_in), 0.5, dtype=torch.float32, device=gpu_device)
+    _gemm_raw(gpu_device, dyg, xg, n_out, n_in, T, 0, 0, g, True, False)
+    assert (g.double().cpu() - (ref + 0.5)).abs().max().item() <= tol, "accumulate"
+    _gemm_raw(gpu_device, dyg, xg, n_out, n_in, T, 0, 0, g, False, False)
+    assert (g.double().cpu() - ref).abs().max().item() <= tol, "overwrite"
+    wide = torch.zeros(n_out, n_in + 2, dtype=torch.float32, device=gpu_device)  # row stride not a multiple of 4: 8-wave kernel
+    g8 = wide[:, :n_in]
+    _gemm_raw(gpu_device, dyg, xg, n_out, n_in, T, 0, 0, g8, False, False)
+    assert torch.equal(g8, g), "4-wave and 8-wave kernels differ"
+    assert float(wide[:, n_in:].abs().max()) == 0.0, "wrote past the output's columns"
+
+
 def test_gemm_linearity_large(K, gpu_device):
     """Size-independent property at a full-size shape: a column block of the result equals the GEMM on that block of W --
     bit for bit where both launches sum in the same order, and to one bf16 ulp on a rare element where the narrow launch
