@@ -7,7 +7,7 @@
 //
 // Layout: rows of h bf16, h % 8 == 0.  Up to h = 8192 a row is held in registers (read from HBM exactly once): forward by
 // TPR = min(256, h/8 rounded up to a wave) threads whose row sums meet through a double-buffered LDS cell; backward by one
-// wave (h <= 4096) or by a pair of waves (wider rows).  Rows up to 32768 wide go through two-pass kernels.
+// wave (h <= 2048), two waves (h <= 4096) or four (wider rows).  Rows up to 32768 wide go through two-pass kernels.
 #include "common.h"
 
 #include <mutex>
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const bf16_t* __restri
 }
 
 // Backward: dx = rstd * (g - xhat * mean(g * xhat)),  g = dy * w, xhat = x * rstd;  dw = sum_rows dy * xhat.
-// ---- backward with one wave per row (h <= 4096) ----------------------------------------------------------------
+// ---- backward with one wave per row (h <= 2048) ----------------------------------------------------------------
 // A row is owned by ONE wave: lane l holds the 8 columns (c * 64 + l) * 8 .. + 7 of chunk c, so every chunk is one
 // coalesced 1 KiB access, the row sums need wave shuffles only and there is no barrier inside the row loop: the waves
 // of a CU run out of step and keep HBM busy while others compute.  Loads and stores carry the streaming hint (in the
@@ -165,23 +165,26 @@ __global__ __launch_bounds__(512) void rmsnorm_bwd_wave_kernel(const bf16_t* __r
     for (int j = threadIdx.x; j < h; j += 512) dw_partial[(size_t)blockIdx.x * h + j] = fold[j];
 }
 
-// ---- backward with two waves per row (4096 < h <= 8192) -------------------------------------------------------------
-// The same scheme with a row shared by the two waves of a pair: wave half 0 owns the first NCHUNK * 512 columns, half 1 the
-// rest, so the per-lane state (operands, weight, dw partials) is that of a row of half the width and stays in registers.
-// The two partial sums of a row meet in an LDS cell (double buffered by iteration parity: one barrier per row).  A block is
-// 4 waves = 2 rows per pass, two blocks per CU: while the waves of one block wait at their barrier the other block's loads
-// are in flight.
-template <int NCHUNK, bool HAS_DRES>
-__global__ __launch_bounds__(256, 2) void rmsnorm_bwd_pair_kernel(const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
-                                                                  const bf16_t* __restrict__ w, const float* __restrict__ rstd,
-                                                                  const bf16_t* __restrict__ dres, bf16_t* __restrict__ dx,
-                                                                  float* __restrict__ dw_partial, int T, int h) {
+// ---- backward with two or four waves per row (2048 < h <= 8192) ---------------------------------------------------
+// The same scheme with a row shared by NSPLIT (2 or 4) waves: wave part p owns NCHUNK * 512 columns from p * NCHUNK * 512
+// on, so the per-lane state (operands, weight, dw partials) is that of a row of 1/NSPLIT of the width, stays in registers
+// and leaves room for a second set of operand registers: the loads of a wave's next row are issued before the current row
+// is worked on, so HBM requests are in flight all the time.  (With one row per wave and nothing prefetched a wave loads,
+// waits, computes and stores in turn, and at T = h = 4096 each wave sees only two rows: 45 us for backward + column sum
+// against 29 us with the prefetch.)  The partial sums of a row meet in an LDS cell (double buffered by iteration parity:
+// one barrier per row).  A block is 4 waves = 4 / NSPLIT rows per pass, two blocks per CU.
+template <int NCHUNK, int NSPLIT, bool HAS_DRES>
+__global__ __launch_bounds__(256, 2) void rmsnorm_bwd_split_kernel(const bf16_t* __restrict__ dy, const bf16_t* __restrict__ x,
+                                                                   const bf16_t* __restrict__ w, const float* __restrict__ rstd,
+                                                                   const bf16_t* __restrict__ dres, bf16_t* __restrict__ dx,
+                                                                   float* __restrict__ dw_partial, int T, int h) {
+    constexpr int RPB = 4 / NSPLIT;  // rows per block pass
     extern __shared__ float fold[];  // h floats
-    __shared__ float cell[2][2][2];  // [parity][row slot][half]
+    __shared__ float cell[2][RPB][NSPLIT];  // [parity][row slot][part]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform values stay in scalar registers
-    const int slot = wave >> 1, half = wave & 1;
-    const int col0 = (half * NCHUNK * 64 + lane) * 8;  // this lane's first column; chunk c is 512 c further
+    const int slot = wave / NSPLIT, part = wave % NSPLIT;
+    const int col0 = (part * NCHUNK * 64 + lane) * 8;  // this lane's first column; chunk c is 512 c further
     bf16x8 wr[NCHUNK];
     float dwacc[NCHUNK][8];
 #pragma unroll
@@ -193,33 +196,48 @@ __global__ __launch_bounds__(256, 2) void rmsnorm_bwd_pair_kernel(const bf16_t* 
     }
     const float inv_h = 1.0f / (float)h;
     int parity = 0;
-    // every wave of the block runs the same number of iterations (barrier inside)
-    for (int row0 = blockIdx.x * 2; row0 < T; row0 += gridDim.x * 2) {
-        const int row = row0 + slot;
+    bf16x8 nxr[NCHUNK], ndyr[NCHUNK], ndrr[NCHUNK];
+    float nrs = 0.f;
+    auto fetch = [&](int row) {  // the operands of this wave's share of `row` into the next-row registers
         const bool live = row < T;
-        const bf16_t* xrow = x + (size_t)row * h + col0;
-        const bf16_t* dyrow = dy + (size_t)row * h + col0;
-        const float rs = live ? rstd[row] : 0.f;
-        bf16x8 xr[NCHUNK], dyr[NCHUNK], drr[NCHUNK];
+        nrs = live ? rstd[row] : 0.f;
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) { xr[c][i] = (bf16_t)0.0f; dyr[c][i] = (bf16_t)0.0f; }
+            for (int i = 0; i < 8; ++i) { nxr[c][i] = (bf16_t)0.0f; ndyr[c][i] = (bf16_t)0.0f; }
             if (live && col0 + c * 512 < h) {
-                xr[c] = ld_bf16x8_nt(xrow + c * 512);
-                dyr[c] = ld_bf16x8_nt(dyrow + c * 512);
-                if (HAS_DRES) drr[c] = ld_bf16x8_nt(dres + (size_t)row * h + col0 + c * 512);
+                nxr[c] = ld_bf16x8_nt(x + (size_t)row * h + col0 + c * 512);
+                ndyr[c] = ld_bf16x8_nt(dy + (size_t)row * h + col0 + c * 512);
+                if (HAS_DRES) ndrr[c] = ld_bf16x8_nt(dres + (size_t)row * h + col0 + c * 512);
             }
         }
+    };
+    fetch(blockIdx.x * RPB + slot);
+    // every wave of the block runs the same number of iterations (barrier inside)
+    for (int row0 = blockIdx.x * RPB; row0 < T; row0 += gridDim.x * RPB) {
+        const int row = row0 + slot;
+        const bool live = row < T;
+        bf16x8 xr[NCHUNK], dyr[NCHUNK], drr[NCHUNK];
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+            xr[c] = nxr[c];
+            dyr[c] = ndyr[c];
+            if (HAS_DRES) drr[c] = ndrr[c];
+        }
+        const float rs = nrs;
+        if (row0 + (int)gridDim.x * RPB < T) fetch(row + gridDim.x * RPB);
         float dot = 0.f;
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c)
 #pragma unroll
             for (int i = 0; i < 8; ++i) dot += (float)dyr[c][i] * (float)wr[c][i] * ((float)xr[c][i] * rs);
         dot = wave_sum(dot);
-        if (lane == 0) cell[parity][slot][half] = dot;
+        if (lane == 0) cell[parity][slot][part] = dot;
         __syncthreads();
-        const float cmean = (cell[parity][slot][0] + cell[parity][slot][1]) * inv_h;  // same order in both waves
+        float rowdot = cell[parity][slot][0];  // same order in every wave of the row
+#pragma unroll
+        for (int q = 1; q < NSPLIT; ++q) rowdot += cell[parity][slot][q];
+        const float cmean = rowdot * inv_h;
         parity ^= 1;
         bf16_t* dxrow = dx + (size_t)row * h + col0;
 #pragma unroll
@@ -239,15 +257,15 @@ __global__ __launch_bounds__(256, 2) void rmsnorm_bwd_pair_kernel(const bf16_t* 
             }
         }
     }
-    for (int s = 0; s < 2; ++s) {  // row slot 0 stores, slot 1 adds: a fixed order
-        if (slot == s) {
+    for (int s2 = 0; s2 < RPB; ++s2) {  // row slot 0 stores, the next adds: a fixed order
+        if (slot == s2) {
 #pragma unroll
             for (int c = 0; c < NCHUNK; ++c) {
                 const int col = col0 + c * 512;
                 if (col < h) {
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
-                        if (s == 0) fold[col + i] = dwacc[c][i];
+                        if (s2 == 0) fold[col + i] = dwacc[c][i];
                         else fold[col + i] += dwacc[c][i];
                     }
                 }
@@ -449,7 +467,11 @@ int rmsnorm_bwd_launch(const void* dy, const void* x, const void* weight, const 
                        hipStream_t st) {
     const size_t smem = (size_t)h * sizeof(float);
     int64_t grid;
-    if (h <= 4096) {  // one wave per row, 8 rows per block
+#define LAUNCH_SPLIT(NC, NS, DR)                                                                                           \
+    hipLaunchKernelGGL((rmsnorm_bwd_split_kernel<NC, NS, DR>), dim3((unsigned)grid), dim3(256), smem, st, (const bf16_t*)dy, \
+                       (const bf16_t*)x, (const bf16_t*)weight, (const float*)rstd, (const bf16_t*)dresidual, (bf16_t*)dx,  \
+                       partials, (int)rows, (int)h)
+    if (h <= 2048) {  // one wave per row, 8 rows per block
         const int nchunk = ((int)h + 511) / 512;
         grid = (rows + 7) / 8;
         if (grid > max_blocks) grid = max_blocks;
@@ -462,13 +484,23 @@ int rmsnorm_bwd_launch(const void* dy, const void* x, const void* weight, const 
     do {                                               \
         if (nchunk <= 1) LAUNCH(1, DR);                \
         else if (nchunk <= 2) LAUNCH(2, DR);           \
-        else if (nchunk <= 4) LAUNCH(4, DR);           \
-        else LAUNCH(8, DR);                            \
+        else LAUNCH(4, DR);                            \
     } while (0)
         if (dresidual) LAUNCH_NC(true); else LAUNCH_NC(false);
 #undef LAUNCH_NC
 #undef LAUNCH
-    } else if (h > 8192) {  // rows that do not fit into registers: two passes per row, dw sums in LDS
+    } else if (h <= 4096) {  // two waves per row (3 or 4 chunks of 512 columns each), 2 rows per block pass
+        grid = (rows + 1) / 2;
+        if (grid > max_blocks) grid = max_blocks;
+        if (grid < 1) grid = 1;
+        if (h <= 3072) { if (dresidual) LAUNCH_SPLIT(3, 2, true); else LAUNCH_SPLIT(3, 2, false); }
+        else { if (dresidual) LAUNCH_SPLIT(4, 2, true); else LAUNCH_SPLIT(4, 2, false); }
+    } else if (h <= 8192) {  // four waves per row, one row per block pass
+        grid = rows < max_blocks ? rows : max_blocks;
+        if (grid < 1) grid = 1;
+        if (h <= 6144) { if (dresidual) LAUNCH_SPLIT(3, 4, true); else LAUNCH_SPLIT(3, 4, false); }
+        else { if (dresidual) LAUNCH_SPLIT(4, 4, true); else LAUNCH_SPLIT(4, 4, false); }
+    } else {  // rows that do not fit into registers: two passes per row, dw sums in LDS
         grid = rows < max_blocks ? rows : max_blocks;
         if (grid < 1) grid = 1;
         if (dresidual)
@@ -477,25 +509,8 @@ int rmsnorm_bwd_launch(const void* dy, const void* x, const void* weight, const 
         else
             hipLaunchKernelGGL(rmsnorm_bwd_wide_kernel<false>, dim3((unsigned)grid), dim3(kWideThreads), 0, st, (const bf16_t*)dy, (const bf16_t*)x,
                                (const bf16_t*)weight, (const float*)rstd, (const bf16_t*)dresidual, (bf16_t*)dx, partials, (int)rows, (int)h);
-    } else {  // wider rows: two waves per row, 2 rows per block pass, two blocks per CU
-        const int nchunk = ((int)h + 1023) / 1024;  // 512-column chunks per wave
-        grid = (rows + 1) / 2;
-        if (grid > max_blocks) grid = max_blocks;
-        if (grid < 1) grid = 1;
-#define LAUNCH(NC, DR)                                                                                                    \
-    hipLaunchKernelGGL((rmsnorm_bwd_pair_kernel<NC, DR>), dim3((unsigned)grid), dim3(256), smem, st, (const bf16_t*)dy,    \
-                       (const bf16_t*)x, (const bf16_t*)weight, (const float*)rstd, (const bf16_t*)dresidual, (bf16_t*)dx, \
-                       partials, (int)rows, (int)h)
-#define LAUNCH_NC(DR)                                  \
-    do {                                               \
-        if (nchunk <= 5) LAUNCH(5, DR);                \
-        else if (nchunk <= 6) LAUNCH(6, DR);           \
-        else LAUNCH(8, DR);                            \
-    } while (0)
-        if (dresidual) LAUNCH_NC(true); else LAUNCH_NC(false);
-#undef LAUNCH_NC
-#undef LAUNCH
     }
+#undef LAUNCH_SPLIT
     EZL_LAUNCH_CHECK("ezl_rmsnorm_bwd");
     hipLaunchKernelGGL(ezl_colsum_kernel<0>, dim3((unsigned)((h + 63) / 64)), dim3(kColsumThreads), 0, st, (const float*)partials,
                        (int)grid, (int)h, (bf16_t*)dw_bf16, (float*)dw_f32, accumulate);
