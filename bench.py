@@ -30,7 +30,7 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak
 # HBM-side bytes per GEMM launch (average over the launches of one step), from two rocprofv3 --pmc runs of this script
 # (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for the streaming kernels of known size in the same
 # run (factor 2.0 for FETCH_SIZE, 1.0 for WRITE_SIZE); see profiles/c2_step_gemm_hbm_traffic.txt.
-GEMM_HBM_BYTES_PER_LAUNCH = {"C2": 601.0e6}
+GEMM_HBM_BYTES_PER_LAUNCH = {"C2": 600.9e6}
 
 
 def cpu_baseline(w, flops):
